@@ -119,10 +119,10 @@ class CacheGroup:
         if device is not None:
             import torch
 
-            n, h, d = len(units), spec.num_kv_heads, spec.head_dim
-            # keys [unit][page][kv head][slot][d]; values transposed [unit][page][kv head][d][slot]
+            n, h, d, dv = len(units), spec.num_kv_heads, spec.head_dim, spec.v_dim
+            # keys [unit][page][kv head][slot][d]; values transposed [unit][page][kv head][dv][slot]
             self.keys = torch.zeros((n, num_pages, h, page_size, d), dtype=torch_dtype, device=device)
-            self.values = torch.zeros((n, num_pages, h, d, page_size), dtype=torch_dtype, device=device)
+            self.values = torch.zeros((n, num_pages, h, dv, page_size), dtype=torch_dtype, device=device)
             self.table = torch.full((max_requests, max_pages_per_request), -1, dtype=torch.int32, device=device)
 
     def poison(self, page: int) -> None:
@@ -131,7 +131,7 @@ class CacheGroup:
             self.values[:, page].fill_(float("nan"))
 
     def bytes_per_token(self, element_size: int) -> int:
-        return 2 * len(self.units) * self.spec.num_kv_heads * self.spec.head_dim * element_size
+        return len(self.units) * self.spec.num_kv_heads * (self.spec.head_dim + self.spec.v_dim) * element_size
 
 
 class GraphStore(dict):
@@ -167,7 +167,8 @@ class CacheManager:
         self.state_units: dict[int, StateSpec] = {}
         for unit, spec in enumerate(unit_specs):
             if isinstance(spec, PagedKVSpec):
-                keyed.setdefault((spec.num_kv_heads, spec.head_dim, spec.window), []).append(unit)
+                keyed.setdefault((spec.num_kv_heads, spec.head_dim, spec.window, spec.value_dim,
+                                  int(spec.keep_first or 0)), []).append(unit)
             elif isinstance(spec, StateSpec):
                 self.state_units[unit] = spec
             elif spec is not None:
@@ -177,8 +178,8 @@ class CacheManager:
             raise ValueError(f"{len(keyed)} cache groups but {len(sizes)} pool sizes")
         self.groups: list[CacheGroup] = []
         self.unit_place: dict[int, tuple[int, int]] = {}
-        for index, ((h, d, window), units) in enumerate(keyed.items()):
-            group = CacheGroup(index, PagedKVSpec(h, d, window), units, sizes[index], page_size, max_requests,
+        for index, ((h, d, window, value_dim, keep_first), units) in enumerate(keyed.items()):
+            group = CacheGroup(index, PagedKVSpec(h, d, window, value_dim, keep_first), units, sizes[index], page_size, max_requests,
                                self.max_pages_per_request, torch_dtype, device)
             self.groups.append(group)
             for position, unit in enumerate(units):
@@ -227,6 +228,13 @@ class CacheManager:
             return 0
         return max(0, next_position - group.spec.window + 1) // self.page_size
 
+    def _kept_pages(self, group: CacheGroup) -> int:
+        """Logical pages at the start of a request that a window never releases (they hold the
+        first tokens that every query keeps seeing)."""
+        if group.spec.window is None or not group.spec.keep_first:
+            return 0
+        return -(-int(group.spec.keep_first) // self.page_size)
+
     def pages_to_reserve(self, request_id: Optional[Hashable], start: int, end: int) -> list[int]:
         """Pages each group must still take so positions ``< end`` are held for a
         step whose first query is at ``start``."""
@@ -235,8 +243,8 @@ class CacheManager:
         for gi, group in enumerate(self.groups):
             needed_to = -(-end // self.page_size)
             have = len(request.groups[gi].pages) if request else 0
-            first = max(have, self._first_needed(group, start))
-            out.append(max(0, needed_to - first))
+            first, kept = self._first_needed(group, start), self._kept_pages(group)
+            out.append(max(0, needed_to - max(have, first)) + max(0, min(kept, first, needed_to) - have))
         return out
 
     def can_reserve(self, request_id: Optional[Hashable], start: int, end: int) -> bool:
@@ -265,10 +273,10 @@ class CacheManager:
         for gi, group in enumerate(self.groups):
             mine = request.groups[gi]
             needed_to = -(-end // self.page_size)
-            first = self._first_needed(group, start)
+            first, kept = self._first_needed(group, start), self._kept_pages(group)
             while len(mine.pages) < needed_to:
                 logical = len(mine.pages)
-                if logical < first:
+                if kept <= logical < first:
                     mine.pages.append(-1)  # never needed: the window starts above it
                     mine.first_held = max(mine.first_held, logical + 1)
                     continue
@@ -286,7 +294,7 @@ class CacheManager:
         for gi, group in enumerate(self.groups):
             mine = request.groups[gi]
             first = min(self._first_needed(group, length), len(mine.pages))
-            for logical in range(mine.first_held, first):
+            for logical in range(max(mine.first_held, self._kept_pages(group)), first):
                 page = mine.pages[logical]
                 if page >= 0:
                     self._release_page(group, page)

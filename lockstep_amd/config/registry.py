@@ -1,7 +1,8 @@
 """One registry from an architecture's name to its typed configuration.
 
-``config.json`` names its architecture twice: ``model_type`` (e.g. ``qwen3``)
-and ``architectures`` (e.g. ``["Qwen3ForCausalLM"]``).  Either name finds the
+``config.json`` names its architecture in ``model_type`` (e.g. ``qwen3``), in
+``architectures`` (e.g. ``["Qwen3ForCausalLM"]``) or in ``architecture`` (one
+name, e.g. ``Bikovik``).  Any of these names finds the
 configuration class; the class turns the file into a ``ModelSpec`` and the
 generic builder in ``lockstep_amd.engine.model`` turns that into a model, so
 registering a configuration class is all that adding an architecture takes.
@@ -41,17 +42,19 @@ def known_architectures() -> list[str]:
 
 
 def config_class_for(raw: Mapping[str, Any]) -> type[ModelConfig]:
-    """The class registered for ``raw["model_type"]`` or ``raw["architectures"]``."""
+    """The class registered for ``raw["model_type"]``, ``raw["architectures"]`` or ``raw["architecture"]``."""
     names = []
     if raw.get("model_type") is not None:
         names.append(raw["model_type"])
     names.extend(raw.get("architectures") or [])
+    if isinstance(raw.get("architecture"), str):
+        names.append(raw["architecture"])
     for name in names:
         if name in _ARCHITECTURES:
             return _ARCHITECTURES[name]
     raise ConfigError(
         f"no architecture is registered for model_type={raw.get('model_type')!r}, "
-        f"architectures={raw.get('architectures')!r}; known: {', '.join(known_architectures()) or 'none'}"
+        f"architectures={raw.get('architectures')!r}, architecture={raw.get('architecture')!r}; known: {', '.join(known_architectures()) or 'none'}"
     )
 
 

@@ -1,0 +1,50 @@
+// The C interface of the mixers library (mixers.hip).  Conventions as in core_api.h: dtype 0 is
+// float32 and 1 bfloat16, pointers are device pointers, `stream` is a hipStream_t passed as
+// void*, the return value is 0 or a negative code whose message ls_last_error() returns.
+#pragma once
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* ls_last_error();
+
+// Dynamic Tanh norm of rows of the float residual stream: h[row] += P[0][row] + P[1][row] + ... first when P
+// [slices][p_rows][width] is given; out [n_rows][ld_out] = tanh(alpha[0] * h[row]) * weight + bias, or nothing
+// when out is null.  rows: the rows of h to take, or null for the first n_rows.
+int ls_dyt(int dtype, float* h, const float* P, int slices, int p_rows, const float* weight, const float* bias,
+           const float* alpha, void* out, const int* rows, int n_rows, int width, long ldh, long ld_out, void* stream);
+
+// x float [rows][2 * width] (gates, then ups): out = g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit),
+// u = clamp(up, -limit, limit).
+int ls_glu_clamped(int out_dtype, const float* x, long ldx, void* out, long ldo, int rows, int width, float limit,
+                   float alpha, void* stream);
+
+// x = cap * tanh(x / cap) in place on float rows.
+int ls_softcap(float* x, long ld, int rows, int width, float cap, void* stream);
+
+// Post pass of an attention projection with keys of size D and values of size DV (see mixers.hip).
+int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int DV, const float* bias,
+                const float* cos_table, const float* sin_table, int rot, int table_positions, int max_pos,
+                const int* tok_seq, const int* tok_pos, const void* seqs, const int* table, int table_stride,
+                void* q_out, long ldq, void* k_pages, void* v_pages, int page_size, int vmix_mode, const float* vmix,
+                float* v_first, long ldv, void* stream);
+
+// Linear recurrence S_t = diag(a_t) S_(t-1) + b_t v_t^T, o_t = S_t^T q_t over the tokens of every request of the
+// step, state [slots][H][D][DV] float (mode 0: HGRN2 gates from p0 = lower bounds [H*D] and p1 = gate bias or null;
+// mode 1: retention with p0 = decay [H] and rotated q, k).  out [T][ldo] float gets o_t.
+int ls_linrec_max_dim();
+int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_at, int v_at, int H, int D, int DV, const float* p0,
+              const float* p1, const float* cos_table, const float* sin_table, int rot, int table_positions,
+              int max_pos, const void* seqs, int n_seqs, float* state, float* out, long ldo, void* stream);
+
+// Per (token, head): x [DV] / sqrt(mean(x^2) + eps), times weight [DV] and silu(gate) where given.
+int ls_head_norm_gate(int out_dtype, const float* x, long ldx, int n_tokens, int H, int DV, const float* weight,
+                      const float* gate, long ldg, float eps, void* out, long ldo, void* stream);
+
+int ls_listed_index(const char* name);
+int ls_call_listed(int index, const long long* words, int n);
+
+#ifdef __cplusplus
+}
+#endif

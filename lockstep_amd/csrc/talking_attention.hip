@@ -1,0 +1,265 @@
+// Attention whose heads talk to each other before the softmax, over the paged cache, with a sliding
+// window that keeps the first tokens, and with keys and values of different sizes:
+//
+//   raw_g[i, j]  = (q_g[i] . k_kv(g)[j]) * scale                  for all query heads g
+//   s_h[i, j]    = sum_g talk[h, g] raw_g[i, j]                   (the heads' scores are mixed)
+//   visible(i,j) = j <= i and (i - j < window or j < keep_first)  (absolute positions)
+//   o_h[i]       = sum_j softmax_j(s_h[i, .])[j] v_kv(h)[j]
+//
+// Because every head's score at a (query, key) pair needs all heads' raw scores there, a workgroup
+// takes a block of 16 query rows of one request with ALL heads, and walks the visible keys in
+// tiles of 32 keys anchored at absolute positions (the kept first tiles, then the window's).  The
+// library is compiled for one shape: LS_TA_HEADS query heads, LS_TA_KV_HEADS key/value heads,
+// keys of LS_TA_DIM and values of LS_TA_VDIM elements, so that the heads' scores and the output
+// accumulators are registers.  The heads are dealt to NW waves.  Per tile:
+//   1. every wave forms the transposed raw scores S^T = K Q^T of its own heads with the MFMA atom
+//      (keys are the first operand, so a lane ends with four consecutive keys of one query row:
+//      the layout in which the probabilities enter the value product) and leaves them in LDS;
+//   2. after a barrier it mixes all heads' raw scores into its own heads' scores (the mixing is
+//      per (query, key) pair, i.e. per lane and register), masks, and runs the online softmax
+//      (row statistics over the four lanes that share a query row);
+//   3. O^T += V^T P^T per head with the atom (value columns are the first operand, so the lane
+//      that holds a row's statistics also holds the row's accumulators).
+// Scores, weights, statistics and accumulators are float; products read the compute dtype T.
+// Keys a request does not hold (beyond its length, pages a window has released) enter as zeros and
+// are masked; their values are replaced by zeros before the product.
+
+#include "common.h"
+
+#ifndef LS_TA_HEADS
+#error "compile with -DLS_TA_HEADS, -DLS_TA_KV_HEADS, -DLS_TA_DIM and -DLS_TA_VDIM"
+#endif
+
+namespace ls {
+
+constexpr int H = LS_TA_HEADS, G = LS_TA_KV_HEADS, D = LS_TA_DIM, DV = LS_TA_VDIM;
+static_assert(H % G == 0, "query heads must be a multiple of the key/value heads");
+static_assert(D % 8 == 0, "key size must be a multiple of 8");
+static_assert(DV % 4 == 0, "value size must be a multiple of 4");
+static_assert(H <= 32, "the heads' raw scores of a tile must fit into LDS");
+constexpr int NW = H % 4 == 0 ? 4 : (H % 2 == 0 ? 2 : 1);  // waves of a workgroup
+constexpr int HPW = H / NW;                                // heads a wave owns
+constexpr int VB = (DV + 15) / 16;                         // blocks of 16 value columns (the last may be partial)
+constexpr int kTileKeys = 32;
+
+struct SeqMeta {
+  int q_off, q_len, q_start, kv_len, table_row, reserved[3];
+};
+
+template <typename T>
+__device__ __forceinline__ typename Atom<T>::vec_t load_or_zero(const T* p, bool ok) {
+  typedef typename Atom<T>::vec_t vec_t;
+  // (an address that is always valid, the value chosen afterwards: the loads of a tile can be in flight together)
+  vec_t v = *reinterpret_cast<const vec_t*>(p);
+  return ok ? v : Atom<T>::zero();
+}
+
+template <typename T>
+__global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
+    const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ blocks,
+    const float* __restrict__ talk, float scale, int window, int keep_first, T* __restrict__ out, long ldo) {
+  constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
+  constexpr int KCH = (D + KC - 1) / KC;  // chunks of a key (lanes beyond D in the last one bring zeros)
+  __shared__ float raw_s[H][2][4][64];  // [head][half of the tile][i][lane]
+  __shared__ float talk_s[H * H];
+  const int seq = blocks[2 * blockIdx.x], rb = blocks[2 * blockIdx.x + 1];
+  const SeqMeta m = seqs[seq];
+  const int row0 = rb * 16;
+  if (row0 >= m.q_len) return;
+  const int nrows = min(16, m.q_len - row0);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4;
+  for (int i = threadIdx.x; i < H * H; i += 64 * NW) talk_s[i] = talk[i];
+  const int p_first = m.q_start + row0, p_last = p_first + nrows - 1;
+  const bool row_ok = l16 < nrows;
+  const int my_pos = p_first + l16;
+  const int* my_table = table + (long)m.table_row * table_stride;
+  const T* q_row = q + (long)(m.q_off + row0 + (row_ok ? l16 : 0)) * ldq;
+
+  float m_run[HPW], l_run[HPW];
+  f32x4 acc[HPW][VB];
+#pragma unroll
+  for (int x = 0; x < HPW; ++x) {
+    m_run[x] = kNegSentinel;
+    l_run[x] = 0.f;
+#pragma unroll
+    for (int b = 0; b < VB; ++b) acc[x][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int lo_tile = max(0, p_first - window + 1) / kTileKeys;
+  const int hi_tile = p_last / kTileKeys;
+  const int kept_tiles = min((keep_first + kTileKeys - 1) / kTileKeys, lo_tile);
+  const int n_tiles = kept_tiles + (hi_tile - lo_tile + 1);
+  __syncthreads();
+
+  for (int step = 0; step < n_tiles; ++step) {
+    const int tile = step < kept_tiles ? step : lo_tile + (step - kept_tiles);
+    const int key0 = tile * kTileKeys;
+    // -- 1. transposed raw scores of the wave's own heads ------------------------------------
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int key = key0 + 16 * half + l16;
+      const int page = key <= p_last ? my_table[key / page_size] : -1;
+      const bool key_ok = page >= 0;
+      const long slot_at = ((long)(key_ok ? page : 0) * G) * page_size + (key_ok ? key % page_size : 0);
+#pragma unroll
+      for (int x = 0; x < HPW; ++x) {
+        const int h = w * HPW + x, g = h / (H / G);
+        const T* k_row = k_pages + (slot_at + (long)g * page_size) * D;
+        f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) {
+          const bool in = c * KC + VEC * quad + VEC <= D;
+          const int at = in ? c * KC + VEC * quad : 0;
+          Atom<T>::mma(s, load_or_zero<T>(k_row + at, key_ok && in), load_or_zero<T>(q_row + h * D + at, row_ok && in));
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) raw_s[h][half][i][lane] = s[i] * scale;
+      }
+    }
+    __syncthreads();
+    // -- 2. mix, mask, online softmax; 3. values ------------------------------------------------
+    bool see[2][4];
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + 16 * half + 4 * quad + i;
+        see[half][i] = row_ok && key <= my_pos && (my_pos - key < window || key < keep_first);
+      }
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) {
+      const int h = w * HPW + x, g = h / (H / G);
+      float s[2][4];
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[half][i] = 0.f;
+      for (int o = 0; o < H; ++o) {
+        const float weight = talk_s[h * H + o];
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s[half][i] = s[half][i] + weight * raw_s[o][half][i][lane];
+      }
+      float top = kNegSentinel;
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) top = fmaxf(top, see[half][i] ? s[half][i] : kNegSentinel);
+      top = quad16_max(top);
+      const float m_new = fmaxf(m_run[x], top);
+      const float shrink = softmax_exp<T>(m_run[x] - m_new);
+      float p[2][4], sum = 0.f;
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          p[half][i] = see[half][i] ? softmax_exp<T>(s[half][i] - m_new) : 0.f;
+          sum = sum + p[half][i];
+        }
+      sum = quad16_sum(sum);
+      l_run[x] = l_run[x] * shrink + sum;
+      m_run[x] = m_new;
+      // values of the tile's keys, value column 16 b + l16, keys 4 quad .. 4 quad + 3 of each half
+      long v_at[2];
+      bool v_ok[2][4];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int key = key0 + 16 * half + 4 * quad;
+        const int page = key <= p_last ? my_table[key / page_size] : -1;
+        v_at[half] = (((long)(page >= 0 ? page : 0) * G + g) * DV) * page_size + (page >= 0 ? key % page_size : 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v_ok[half][i] = page >= 0 && key + i <= p_last;
+      }
+#pragma unroll
+      for (int b = 0; b < VB; ++b) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[x][b][i] = acc[x][b][i] * shrink;
+        const bool col_ok = 16 * b + l16 < DV;
+        const long column = (long)(col_ok ? 16 * b + l16 : 0) * page_size;
+        if constexpr (sizeof(T) == 2) {
+          const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[0] + column);
+          const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[1] + column);
+          bf16x8 a, pb;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            a[i] = (v_ok[0][i] && col_ok) ? v0[i] : (bf16_t)0.f;
+            a[4 + i] = (v_ok[1][i] && col_ok) ? v1[i] : (bf16_t)0.f;
+            pb[i] = (bf16_t)p[0][i];
+            pb[4 + i] = (bf16_t)p[1][i];
+          }
+          Atom<T>::mma(acc[x][b], a, pb);
+        } else {
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(v_pages + v_at[half] + column);
+            f32x4 a, pb;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              a[i] = (v_ok[half][i] && col_ok) ? v[i] : 0.f;
+              pb[i] = p[half][i];
+            }
+            Atom<T>::mma(acc[x][b], a, pb);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (!row_ok) return;
+  T* dst = out + (long)(m.q_off + row0 + l16) * ldo;
+#pragma unroll
+  for (int x = 0; x < HPW; ++x) {
+    const int h = w * HPW + x;
+    const float inv = 1.0f / l_run[x];
+#pragma unroll
+    for (int b = 0; b < VB; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (16 * b + 4 * quad + i < DV) dst[h * DV + 16 * b + 4 * quad + i] = from_f32<T>(acc[x][b][i] * inv);
+  }
+}
+
+}  // namespace ls
+
+LS_DEFINE_ERROR_API
+
+using namespace ls;
+
+extern "C" int ls_talk_heads() { return H; }
+extern "C" int ls_talk_kv_heads() { return G; }
+extern "C" int ls_talk_dim() { return D; }
+extern "C" int ls_talk_vdim() { return DV; }
+
+// q [T][ldq] (rotated queries, H heads of D); key pages [pages][G][page_size][D], value pages
+// [pages][G][DV][page_size]; table [slots][table_stride]; seqs: the step's requests; blocks: n_blocks pairs
+// (request of the step, block of 16 of its rows); talk [H][H] float; out [T][ldo] (H heads of DV).
+extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages,
+                                 int page_size, const int* table, int table_stride, const void* seqs,
+                                 const int* blocks, int n_blocks, const float* talk, float scale, int window,
+                                 int keep_first, void* out, long ldo, void* stream) {
+  LS_REQUIRE(n_blocks > 0 && q && k_pages && v_pages && table && seqs && blocks && talk && out, "talk_attention: null operand");
+  LS_REQUIRE(ldq >= (long)H * D && ldo >= (long)H * DV, "talk_attention: rows are too short");
+  LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && table_stride > 0, "talk_attention: page size %d", page_size);
+  LS_REQUIRE(window > 0 && keep_first >= 0, "talk_attention: window %d, kept first tokens %d", window, keep_first);
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(v_pages) % 16 == 0,
+             "talk_attention: operands must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == kF32) {
+    LS_REQUIRE(ldq % 4 == 0, "talk_attention: query rows must be 16-byte aligned");
+    hipLaunchKernelGGL(talk_attention_kernel<float>, dim3(n_blocks), dim3(64 * NW), 0, s, (const float*)q, ldq,
+                       (const float*)k_pages, (const float*)v_pages, page_size, table, table_stride,
+                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (float*)out, ldo);
+  } else if (dtype == kBF16) {
+    LS_REQUIRE(ldq % 8 == 0, "talk_attention: query rows must be 16-byte aligned");
+    hipLaunchKernelGGL(talk_attention_kernel<bf16_t>, dim3(n_blocks), dim3(64 * NW), 0, s, (const bf16_t*)q, ldq,
+                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_size, table, table_stride,
+                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (bf16_t*)out, ldo);
+  } else {
+    return fail("talk_attention: unknown dtype %d", dtype);
+  }
+  return check_launch("talk_attention");
+}

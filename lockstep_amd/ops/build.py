@@ -6,7 +6,11 @@ Two kinds of library exist:
                     (matrix products, norms, rotation and cache write, SwiGLU,
                     embedding, arg-max);
 ``attention<D>``    the attention kernels for one head size ``D``; a model
-                    needs only its own.
+                    needs only its own;
+``mixers``          Dynamic Tanh norm, clamped gated unit, soft cap, the linear
+                    recurrence with per-row gates and what surrounds it;
+``talking<shape>``  attention whose heads' scores are mixed before the softmax,
+                    for one shape (query heads, kv heads, key and value size).
 
 A library's file name carries a hash of its sources and flags, so a stale
 build is never loaded.  Libraries are written next to the package
@@ -39,6 +43,8 @@ FLAGS = [
 ]
 CORE_SOURCES = ("core.hip", "gemm.hip", "sample.hip")
 ATTENTION_SOURCES = ("attention.hip",)
+MIXERS_SOURCES = ("mixers.hip",)
+TALKING_SOURCES = ("talking_attention.hip",)
 
 
 class BuildError(RuntimeError):
@@ -195,6 +201,22 @@ def build_attention(head_dim: int, force: bool = False) -> Path:
     return build(f"attention{head_dim}", ATTENTION_SOURCES, (f"-DLS_HEAD_DIM={head_dim}",), force)
 
 
+def build_mixers(force: bool = False) -> Path:
+    return build("mixers", MIXERS_SOURCES, (), force)
+
+
+def build_talking(heads: int, kv_heads: int, dim: int, vdim: int, force: bool = False) -> Path:
+    """The talking-heads attention library of one shape."""
+    if heads <= 0 or kv_heads <= 0 or heads % kv_heads or heads > 32:
+        raise BuildError(f"{heads} query heads over {kv_heads} key/value heads are not supported: the talking-heads "
+                         "attention kernel takes up to 32 heads, a multiple of the key/value heads")
+    if dim % 8 or not 8 <= dim <= 256 or vdim % 4 or not 4 <= vdim <= 256:
+        raise BuildError(f"key size {dim} / value size {vdim} are not supported: multiples of 8 / of 4, up to 256")
+    return build(f"talking{heads}x{kv_heads}x{dim}x{vdim}", TALKING_SOURCES,
+                 (f"-DLS_TA_HEADS={heads}", f"-DLS_TA_KV_HEADS={kv_heads}", f"-DLS_TA_DIM={dim}",
+                  f"-DLS_TA_VDIM={vdim}"), force)
+
+
 MUTANT_DEFINE = "-DLS_MUTANTS"
 
 
@@ -210,12 +232,18 @@ def build_attention_mutants(head_dim: int, force: bool = False) -> Path:
 
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
 MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the controls
+#: (query heads, kv heads, key size, value size) of the talking-heads attention the tests and measurements use
+DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 4, 128, 128), (32, 8, 128, 128))
 
 
-def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True) -> list[Path]:
-    """Compile the core library and the attention library of each head size,
-    a few at a time; with ``mutants`` also the control libraries of the tests."""
-    jobs = [lambda: build_core(force)] + [lambda d=d: build_attention(d, force) for d in head_dims]
+def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True,
+              talking_shapes=DEFAULT_TALKING_SHAPES) -> list[Path]:
+    """Compile the core library, the mixers library, the attention library of each head size and the
+    talking-heads attention library of each shape, a few at a time; with ``mutants`` also the control
+    libraries of the tests."""
+    jobs = [lambda: build_core(force), lambda: build_mixers(force)]
+    jobs += [lambda d=d: build_attention(d, force) for d in head_dims]
+    jobs += [lambda shape=shape: build_talking(*shape, force) for shape in talking_shapes]
     if mutants:
         jobs += [lambda: build_core_mutants(force)] + [lambda d=d: build_attention_mutants(d, force)
                                                        for d in MUTANT_HEAD_DIMS]

@@ -79,6 +79,10 @@ class Kernels:
         self.core.ls_sample_scratch_bytes.restype = ctypes.c_long
         self._attention: dict[int, ctypes.CDLL] = {}
         self.attention_paths: dict[int, str] = {}
+        self._mixers = None
+        self.mixers_path = None
+        self._talking: dict[tuple, ctypes.CDLL] = {}
+        self.talking_paths: dict[tuple, str] = {}
         self._argmax_scratch: dict = {}
         self._sample_scratch: dict = {}
         self._sample_scratch_kept: list = []
@@ -323,7 +327,8 @@ class Kernels:
             c_long(ld_out), c_float(eps), _stream()))
 
     # -- rows -------------------------------------------------------------------
-    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+        """``out[t] = table[tokens[t]] * scale`` as float32 rows."""
         if not (tokens.is_cuda and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.is_contiguous()):
             raise KernelError("embed tokens must be a contiguous int32 vector on the GPU")
         _rows_ok(table, "embed table"); _rows_ok(out, "embed out")
@@ -335,7 +340,7 @@ class Kernels:
             return
         self._launch(self.core, self.core.ls_embed, (
             c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(table), _ptr(out), c_int(tokens.shape[0]),
-            c_int(table.shape[0]), c_int(table.shape[1]), c_long(out.stride(0)), _stream()))
+            c_int(table.shape[0]), c_int(table.shape[1]), c_long(out.stride(0)), c_float(scale), _stream()))
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float,
                 rows: torch.Tensor | None = None) -> None:
@@ -653,6 +658,240 @@ class Kernels:
         self._launch(lib, lib.ls_attention_combine, (
             c_int(DTYPE_CODE[out.dtype]), _ptr(seqs), _ptr(items), c_int(n_items), c_int(nkv), _ptr(part_acc),
             _ptr(part_ml), _ptr(out), c_long(out.stride(0)), c_int(nq // nkv), c_int(max_rows), _stream()))
+
+    # -- mixers beyond softmax attention: norms, gated units, recurrences ----------------
+    def mixers_lib(self):
+        """The library of csrc/mixers.hip, built and loaded when a part first asks for it."""
+        if self._mixers is None:
+            self.mixers_path = _build.build_mixers()
+            lib = ctypes.CDLL(str(self.mixers_path))
+            lib.ls_last_error.restype = ctypes.c_char_p
+            self._mixers = lib
+        return self._mixers
+
+    def talking_lib(self, heads: int, kv_heads: int, dim: int, vdim: int):
+        """The talking-heads attention library of one shape."""
+        shape = (heads, kv_heads, dim, vdim)
+        lib = self._talking.get(shape)
+        if lib is None:
+            path = _build.build_talking(*shape)
+            lib = ctypes.CDLL(str(path))
+            lib.ls_last_error.restype = ctypes.c_char_p
+            if (lib.ls_talk_heads(), lib.ls_talk_kv_heads(), lib.ls_talk_dim(), lib.ls_talk_vdim()) != shape:
+                raise KernelError(f"{path} was built for another shape")
+            self._talking[shape] = lib
+            self.talking_paths[shape] = str(path)
+        return lib
+
+    @staticmethod
+    def _f32_vector(t, n: int, name: str) -> None:
+        if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n):
+            raise KernelError(f"{name} must be float32 with {n} elements on the GPU")
+
+    def dyt(self, h: torch.Tensor, weight, bias, alpha, out, rows: torch.Tensor | None = None,
+            partials: torch.Tensor | None = None) -> None:
+        """Dynamic Tanh norm: ``out = tanh(alpha * h[row]) * weight + bias`` on rows of the float32 stream
+        ``h`` (all, or those listed in ``rows``); with ``partials [slices, rows, width]`` these are added
+        to ``h`` first, in ascending order.  ``out`` None: the addition only."""
+        _rows_ok(h, "dyt h")
+        if not (h.dtype == torch.float32):
+            raise KernelError("dyt reads the float32 residual stream")
+        width = h.shape[1]
+        n_rows = h.shape[0] if rows is None else rows.shape[0]
+        if rows is not None and not (rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous()):
+            raise KernelError("dyt rows: int32 on the GPU")
+        slices = p_rows = 0
+        if partials is not None:
+            if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
+                    and partials.dim() == 3 and partials.shape[2] == width and partials.shape[1] >= (h.shape[0] if rows is None else 1)):
+                raise KernelError("dyt partials [slices, rows, width] float32")
+            slices, p_rows = partials.shape[0], partials.shape[1]
+        dtype, ld_out = torch.float32, 0
+        if out is not None:
+            _rows_ok(out, "dyt out")
+            if not (out.dtype in DTYPE_CODE and out.shape == (n_rows, width)):
+                raise KernelError(f"dyt out must be [{n_rows},{width}]")
+            self._f32_vector(weight, width, "dyt weight"); self._f32_vector(bias, width, "dyt bias")
+            self._f32_vector(alpha, 1, "dyt alpha")
+            dtype, ld_out = out.dtype, out.stride(0)
+        if n_rows == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_dyt, (
+            c_int(DTYPE_CODE[dtype]), _ptr(h), _ptr(partials), c_int(slices), c_int(p_rows), _ptr(weight), _ptr(bias),
+            _ptr(alpha), _ptr(out), _ptr(rows), c_int(n_rows), c_int(width), c_long(h.stride(0)), c_long(ld_out),
+            _stream()))
+
+    def glu_clamped(self, x: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> None:
+        """``out = g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit,
+        limit)``; ``x`` float32 ``[rows, 2 * width]`` holds the gates, then the ups."""
+        _rows_ok(x, "glu_clamped x"); _rows_ok(out, "glu_clamped out")
+        rows, width = out.shape
+        if not (x.dtype == torch.float32 and x.shape == (rows, 2 * width) and out.dtype in DTYPE_CODE):
+            raise KernelError(f"glu_clamped reads float32 [{rows},{2 * width}]")
+        if rows == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_glu_clamped, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(x), c_long(x.stride(0)), _ptr(out), c_long(out.stride(0)), c_int(rows),
+            c_int(width), c_float(limit), c_float(alpha), _stream()))
+
+    def softcap(self, x: torch.Tensor, cap: float) -> None:
+        """``x = cap * tanh(x / cap)`` in place on float32 rows."""
+        _rows_ok(x, "softcap x")
+        if not (x.dtype == torch.float32 and cap > 0):
+            raise KernelError("softcap works on float32 rows with a positive cap")
+        if x.shape[0] == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_softcap, (_ptr(x), c_long(x.stride(0)), c_int(x.shape[0]), c_int(x.shape[1]),
+                                           c_float(cap), _stream()))
+
+    @staticmethod
+    def _rotation_tables(cos, sin, rot: int, max_pos: int) -> int:
+        if rot == 0:
+            return 0
+        if not (cos is not None and sin is not None and cos.shape == sin.shape and cos.dim() == 2
+                and cos.shape[1] * 2 == rot and cos.dtype == torch.float32 and sin.dtype == torch.float32
+                and cos.is_contiguous() and sin.is_contiguous() and cos.is_cuda):
+            raise KernelError("rotation tables must be float32 [positions, rotary_dim/2]")
+        if not (max_pos < cos.shape[0]):
+            raise KernelError(f"position {max_pos} is beyond the rotation tables ({cos.shape[0]})")
+        return cos.shape[0]
+
+    def _paged_ok(self, k_pages, v_pages, table, dtype, kv_heads: int, page_size: int, dim: int, vdim: int) -> None:
+        if not (k_pages.dtype == dtype and v_pages.dtype == dtype and k_pages.is_contiguous() and v_pages.is_contiguous()
+                and k_pages.dim() == 4 and k_pages.shape[1:] == (kv_heads, page_size, dim)
+                and v_pages.shape[1:] == (kv_heads, vdim, page_size) and k_pages.shape[0] == v_pages.shape[0]):
+            raise KernelError(f"cache pages do not have the layout [pages,{kv_heads},{page_size},{dim}] / "
+                              f"[pages,{kv_heads},{vdim},{page_size}] of the compute dtype")
+        if not (table.is_cuda and table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous()):
+            raise KernelError("block table must be a contiguous int32 matrix")
+
+    def talk_qkv(self, raw: torch.Tensor, n_tokens: int, heads: int, kv_heads: int, dim: int, vdim: int, bias, cos, sin,
+                 rot: int, max_pos: int, tok_seq, tok_pos, seqs, table, q_out: torch.Tensor, k_pages, v_pages,
+                 page_size: int, vmix_mode: int = 0, vmix=None, v_first=None) -> None:
+        """Post pass of the fused projection ``raw`` (float32 ``[T, heads*dim + kv_heads*dim + kv_heads*vdim]``):
+        biases, rotation of queries and keys, value mixing (1: keep the values in ``v_first``; 2: mix
+        ``v_first`` in with the weight ``vmix``), queries to ``q_out``, keys and values to their pages."""
+        _rows_ok(raw, "talk_qkv raw"); _rows_ok(q_out, "talk_qkv q_out")
+        width = heads * dim + kv_heads * (dim + vdim)
+        if not (raw.dtype == torch.float32 and raw.shape[0] >= n_tokens and raw.shape[1] == width):
+            raise KernelError(f"talk_qkv raw must be float32 [>= {n_tokens}, {width}]")
+        if not (q_out.dtype in DTYPE_CODE and q_out.shape[0] >= n_tokens and q_out.shape[1] == heads * dim):
+            raise KernelError("talk_qkv q_out has the wrong shape or dtype")
+        if bias is not None:
+            self._f32_vector(bias, width, "talk_qkv bias")
+        positions = self._rotation_tables(cos, sin, rot, max_pos)
+        self._paged_ok(k_pages, v_pages, table, q_out.dtype, kv_heads, page_size, dim, vdim)
+        if not (max_pos // page_size < table.shape[1]):
+            raise KernelError(f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
+        for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+            if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n_tokens):
+                raise KernelError(f"{name} must be int32 with at least {n_tokens} entries")
+        ldv = 0
+        if vmix_mode:
+            if not (v_first is not None and v_first.is_cuda and v_first.dtype == torch.float32 and v_first.dim() == 2
+                    and v_first.stride(1) == 1 and v_first.shape[0] >= n_tokens and v_first.shape[1] == kv_heads * vdim):
+                raise KernelError(f"talk_qkv v_first must be float32 [>= {n_tokens}, {kv_heads * vdim}]")
+            ldv = v_first.stride(0)
+            if vmix_mode == 2:
+                self._f32_vector(vmix, 1, "talk_qkv vmix")
+        if n_tokens == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_talk_qkv, (
+            c_int(DTYPE_CODE[q_out.dtype]), _ptr(raw), c_long(raw.stride(0)), c_int(n_tokens), c_int(heads),
+            c_int(kv_heads), c_int(dim), c_int(vdim), _ptr(bias), _ptr(cos), _ptr(sin), c_int(rot), c_int(positions),
+            c_int(max_pos), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table), c_int(table.shape[1]), _ptr(q_out),
+            c_long(q_out.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size), c_int(vmix_mode), _ptr(vmix),
+            _ptr(v_first), c_long(ldv), _stream()))
+
+    def talk_attention(self, q: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, k_pages, v_pages,
+                       page_size: int, table, seqs, blocks: torch.Tensor, n_blocks: int, talk: torch.Tensor,
+                       scale: float, window: int, keep_first: int, out: torch.Tensor) -> None:
+        """Talking-heads attention of the step's queries ``q [T, heads*dim]`` over the paged cache; ``blocks``
+        lists ``n_blocks`` pairs (request of the step, block of 16 of its rows); ``talk [heads, heads]``."""
+        lib = self.talking_lib(heads, kv_heads, dim, vdim)
+        _rows_ok(q, "talk_attention q"); _rows_ok(out, "talk_attention out")
+        if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype and q.shape[1] == heads * dim
+                and out.shape[1] == heads * vdim and out.shape[0] == q.shape[0]):
+            raise KernelError("talk_attention q / out have the wrong shape or dtype")
+        self._paged_ok(k_pages, v_pages, table, q.dtype, kv_heads, page_size, dim, vdim)
+        if not (blocks.is_cuda and blocks.dtype == torch.int32 and blocks.is_contiguous() and blocks.numel() >= 2 * n_blocks):
+            raise KernelError("talk_attention blocks must hold two int32 each")
+        self._f32_vector(talk, heads * heads, "talk_attention talk")
+        if not (window > 0 and keep_first >= 0):
+            raise KernelError(f"talk_attention window {window} / kept first tokens {keep_first}")
+        if n_blocks == 0:
+            return
+        self._launch(lib, lib.ls_talk_attention, (
+            c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
+            _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(blocks), c_int(n_blocks), _ptr(talk), c_float(scale),
+            c_int(window), c_int(keep_first), _ptr(out), c_long(out.stride(0)), _stream()))
+
+    LINREC_HGRN2, LINREC_RETENTION = 0, 1
+
+    def linrec_max_dim(self) -> int:
+        return self._memo(("linrec_max_dim",), lambda: int(self.mixers_lib().ls_linrec_max_dim()))
+
+    def linrec(self, mode: int, raw: torch.Tensor, q_at: int, ab_at: int, v_at: int, heads: int, dim: int, vdim: int,
+               p0, p1, cos, sin, rot: int, max_pos: int, seqs, n_seqs: int, state: torch.Tensor,
+               out: torch.Tensor) -> None:
+        """The linear recurrence ``S_t = diag(a_t) S_(t-1) + b_t v_t^T``, ``o_t = S_t^T q_t`` over the tokens of
+        every request of the step; ``raw`` float32 holds the projections (q at column ``q_at``, the gate or key
+        projection at ``ab_at``, v at ``v_at``), ``state`` float32 ``[slots, heads, dim, vdim]`` is read and
+        left for the next step, ``out`` float32 ``[T, heads*vdim]`` gets ``o_t``.  Mode ``LINREC_HGRN2``:
+        ``p0`` lower bounds ``[heads*dim]``, ``p1`` the gate's bias or None; ``LINREC_RETENTION``: ``p0`` the
+        heads' decays, rotation tables for q and k."""
+        _rows_ok(raw, "linrec raw"); _rows_ok(out, "linrec out")
+        if not (raw.dtype == torch.float32 and out.dtype == torch.float32 and out.shape[1] == heads * vdim
+                and out.shape[0] == raw.shape[0]):
+            raise KernelError("linrec reads and writes float32 rows, out [T, heads*vdim]")
+        if not (0 <= q_at and q_at + heads * dim <= raw.shape[1] and 0 <= ab_at and ab_at + heads * dim <= raw.shape[1]
+                and 0 <= v_at and v_at + heads * vdim <= raw.shape[1]):
+            raise KernelError("linrec: the projections do not fit the rows of raw")
+        if not (dim <= self.linrec_max_dim()):
+            raise KernelError(f"linrec takes states of at most {self.linrec_max_dim()} rows, got {dim}")
+        if not (state.is_cuda and state.dtype == torch.float32 and state.is_contiguous()
+                and tuple(state.shape[1:]) == (heads, dim, vdim)):
+            raise KernelError(f"linrec state must be float32 [slots,{heads},{dim},{vdim}]")
+        positions = 0
+        if mode == self.LINREC_HGRN2:
+            self._f32_vector(p0, heads * dim, "linrec lower bounds")
+            if p1 is not None:
+                self._f32_vector(p1, heads * dim, "linrec gate bias")
+        else:
+            self._f32_vector(p0, heads, "linrec decays")
+            positions = self._rotation_tables(cos, sin, rot, max_pos)
+        if n_seqs == 0 or raw.shape[0] == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_linrec, (
+            c_int(mode), _ptr(raw), c_long(raw.stride(0)), c_int(q_at), c_int(ab_at), c_int(v_at), c_int(heads),
+            c_int(dim), c_int(vdim), _ptr(p0), _ptr(p1), _ptr(cos), _ptr(sin), c_int(rot), c_int(positions),
+            c_int(max_pos), _ptr(seqs), c_int(n_seqs), _ptr(state), _ptr(out), c_long(out.stride(0)), _stream()))
+
+    def head_norm_gate(self, x: torch.Tensor, heads: int, vdim: int, weight, gate, eps: float, out: torch.Tensor) -> None:
+        """Per (token, head): ``x / sqrt(mean(x^2) + eps)`` over the head's ``vdim`` values, times ``weight
+        [vdim]`` and ``silu(gate)`` (float32 rows like ``x``) where given; ``x`` float32 ``[T, heads*vdim]``."""
+        _rows_ok(x, "head_norm_gate x"); _rows_ok(out, "head_norm_gate out")
+        if not (x.dtype == torch.float32 and x.shape[1] == heads * vdim and out.shape == x.shape and out.dtype in DTYPE_CODE):
+            raise KernelError("head_norm_gate reads float32 [T, heads*vdim] and writes the same shape")
+        if weight is not None:
+            self._f32_vector(weight, vdim, "head_norm_gate weight")
+        ldg = 0
+        if gate is not None:
+            if not (gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and gate.stride(1) == 1
+                    and gate.shape == x.shape):
+                raise KernelError("head_norm_gate gate must be float32 rows of the shape of x")
+            ldg = gate.stride(0)
+        if x.shape[0] == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_head_norm_gate, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(x), c_long(x.stride(0)), c_int(x.shape[0]), c_int(heads), c_int(vdim),
+            _ptr(weight), _ptr(gate), c_long(ldg), c_float(eps), _ptr(out), c_long(out.stride(0)), _stream()))
 
 
 ATTENTION_ITEM_INTS = 32

@@ -243,7 +243,7 @@ def tile_page_ids(ctx, coop, nkv: int, head_dim: int, window: int, tile: int):
     None if no group has them."""
     cache, page_size = ctx.cache, ctx.cache.page_size
     group = next((g for g in cache.groups if (g.spec.num_kv_heads, g.spec.head_dim, g.spec.window or 0)
-                  == (nkv, head_dim, window)), None)
+                  == (nkv, head_dim, window) and g.spec.value_dim is None and not g.spec.keep_first), None)
     if group is None:
         return None
     per_tile = tile // page_size

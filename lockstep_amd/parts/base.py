@@ -60,11 +60,19 @@ class WeightSpec:
 
 @dataclass(frozen=True)
 class PagedKVSpec:
-    """Keys and values of every token, or of the last ``window`` tokens."""
+    """Keys and values of every token, or of the last ``window`` tokens; with ``keep_first`` the
+    first that many tokens stay as well when the window has passed them.  ``value_dim``: the size
+    of a value where it differs from the size of a key (``head_dim``)."""
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+    keep_first: int = 0
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
@@ -268,6 +276,24 @@ def deferred_rows(ctx, k: int, n: int) -> int:
     if kernels.gemm_slices_count(k) * n > DEFER_MANY_ROWS_SUMS:
         return min(DEFER_ADD_ROWS, 64)
     return min(DEFER_ADD_ROWS, kernels.gemm_slices_max_rows(k, ctx.rt.dtype))
+
+
+def project_out(ctx, x, weight, out, accumulate: bool, defer: bool, name: str):
+    """A mixer's output projection ``out (+)= x @ weight.T`` into the float32 stream.  With ``defer`` a
+    small step leaves the product as the sums of its K slices for the next reader of the stream
+    (a ``PendingAdd`` is returned), which cuts the work over K as well; else None."""
+    from ..ops import ADD_F32, STORE_F32
+
+    k = ctx.rt.kernels
+    inner = weight.shape[1]
+    if defer and accumulate and 0 < ctx.n_tokens <= deferred_rows(ctx, inner, out.shape[1]):
+        slices = k.gemm_slices_count(inner)
+        partials = ctx.buf(name, (slices * ctx.n_tokens, out.shape[1]), __import__("torch").float32)
+        partials = partials.view(slices, ctx.n_tokens, out.shape[1])
+        k.gemm_slices(x, weight, partials)
+        return PendingAdd(partials)
+    k.gemm(x, weight, out, ADD_F32 if accumulate else STORE_F32)
+    return None
 
 
 def graph_safe_tree(part: Part) -> bool:

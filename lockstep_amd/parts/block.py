@@ -12,7 +12,7 @@ class PreNormResidual(Arrangement):
 
     Parameters name the parts' tensor prefixes below the layer's prefix:
     ``mixer_prefix``, ``feed_forward_prefix``, ``mixer_norm_name``,
-    ``feed_forward_norm_name``.
+    ``feed_forward_norm_name``.  A layer without a ``feed_forward`` part is the first half alone.
     """
 
     graph_safe = True
@@ -24,16 +24,18 @@ class PreNormResidual(Arrangement):
         base = layer_spec.prefix
         self.mixer_norm = build_part(layer_spec.part("mixer_norm"), self.join(base, p["mixer_norm_name"]))
         self._mixer = build_part(layer_spec.part("mixer"), self.join(base, p["mixer_prefix"]))
-        self.feed_forward_norm = build_part(layer_spec.part("feed_forward_norm"),
-                                            self.join(base, p["feed_forward_norm_name"]))
-        self.feed_forward = build_part(layer_spec.part("feed_forward"), self.join(base, p["feed_forward_prefix"]))
+        self.feed_forward = self.feed_forward_norm = None
+        if layer_spec.has("feed_forward"):
+            self.feed_forward_norm = build_part(layer_spec.part("feed_forward_norm"),
+                                                self.join(base, p["feed_forward_norm_name"]))
+            self.feed_forward = build_part(layer_spec.part("feed_forward"), self.join(base, p["feed_forward_prefix"]))
         self._fuse_mixer = self._fuses(self._mixer, self.mixer_norm)
-        self._fuse_ff = self._fuses(self.feed_forward, self.feed_forward_norm)
+        self._fuse_ff = self.feed_forward is not None and self._fuses(self.feed_forward, self.feed_forward_norm)
         # parts that can leave their residual addition to the next norm (see PendingAdd)
         self._defer_mixer = takes(self._mixer.forward, "defer")
-        self._defer_ff = takes(self.feed_forward.forward, "defer")
+        self._defer_ff = self.feed_forward is not None and takes(self.feed_forward.forward, "defer")
         self._norm1_pending = takes(self.mixer_norm.forward, "pending")
-        self._norm2_pending = takes(self.feed_forward_norm.forward, "pending")
+        self._norm2_pending = self.feed_forward is not None and takes(self.feed_forward_norm.forward, "pending")
 
     @classmethod
     def weight_specs(cls, layer_spec, prefix: str = ""):
@@ -42,14 +44,20 @@ class PreNormResidual(Arrangement):
         p = layer_spec.arrangement.params
         base = layer_spec.prefix
         out = []
-        for spec, name in ((layer_spec.part("mixer_norm"), p["mixer_norm_name"]),
-                           (layer_spec.part("mixer"), p["mixer_prefix"]),
-                           (layer_spec.part("feed_forward_norm"), p["feed_forward_norm_name"]),
-                           (layer_spec.part("feed_forward"), p["feed_forward_prefix"])):
+        wired = [(layer_spec.part("mixer_norm"), p["mixer_norm_name"]), (layer_spec.part("mixer"), p["mixer_prefix"])]
+        if layer_spec.has("feed_forward"):
+            wired += [(layer_spec.part("feed_forward_norm"), p["feed_forward_norm_name"]),
+                      (layer_spec.part("feed_forward"), p["feed_forward_prefix"])]
+        elif layer_spec.has("feed_forward_norm"):
+            # a norm the checkpoint may hold although nothing follows it: its tensors are accepted, never used
+            wired.append((layer_spec.part("feed_forward_norm"), p["feed_forward_norm_name"]))
+        for spec, name in wired:
             out += part_class(spec.kind).weight_specs(spec, cls.join(base, name))
         return out
 
     def parts(self):
+        if self.feed_forward is None:
+            return (self.mixer_norm, self._mixer)
         return (self.mixer_norm, self._mixer, self.feed_forward_norm, self.feed_forward)
 
     @property
@@ -94,6 +102,8 @@ class PreNormResidual(Arrangement):
             else:
                 mixed = self._mixer.forward(ctx, run, x, h, accumulate=True)
         mixed = mixed if isinstance(mixed, PendingAdd) else None
+        if self.feed_forward is None:
+            return mixed
         if mixed is not None and (small and self._fuse_ff or not self._norm2_pending):
             mixed.flush(ctx, h)
             mixed = None

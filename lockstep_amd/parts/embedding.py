@@ -9,14 +9,16 @@ from .base import Part, WeightSpec, register_part
 
 @register_part("token_embedding")
 class TokenEmbedding(Part):
-    """``h[t] = E[token[t]]``, no scaling (reference engine/model/qwen3.py:319).
-    Parameters: ``name``, ``vocab_size``, ``hidden_size``."""
+    """``h[t] = E[token[t]] * scale``; without ``scale`` no scaling (reference
+    engine/model/qwen3.py:319).  Parameters: ``name``, ``vocab_size``, ``hidden_size``,
+    ``scale`` (optional)."""
 
     graph_safe = True
 
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
         self.table = None
+        self.scale = float(spec.params.get("scale", 1.0))
 
     @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
@@ -26,15 +28,16 @@ class TokenEmbedding(Part):
         self.table = rt.matrix(weights.get(self.spec["name"]), share_key=weights.source_name(self.spec["name"]))
 
     def forward(self, ctx, tokens, out) -> None:
-        ctx.rt.kernels.embed(tokens, self.table, out)
+        ctx.rt.kernels.embed(tokens, self.table, out, self.scale)
 
 
 @register_part("linear_head")
 class LinearHead(Part):
     """``logits = x @ W^T`` in float32, no bias and no scaling (reference
-    engine/model/qwen3.py:373).  Parameters: ``name``, ``tied_to`` (a tensor
-    name the head aliases when the checkpoint does not hold its own, or None),
-    ``vocab_size``, ``hidden_size``."""
+    engine/model/qwen3.py:373); with ``softcap`` (optional, a positive number c) the
+    logits are then bent into (-c, c): ``c * tanh(logits / c)``.  Parameters: ``name``,
+    ``tied_to`` (a tensor name the head aliases when the checkpoint does not hold its
+    own, or None), ``vocab_size``, ``hidden_size``, ``softcap``."""
 
     graph_safe = True
 
@@ -42,6 +45,10 @@ class LinearHead(Part):
         super().__init__(spec, prefix)
         self.weight = None
         self.vocab = int(spec["vocab_size"])
+        cap = spec.params.get("softcap")
+        self.softcap = float(cap) if cap else None
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError(f"the logits' soft cap must be positive, got {cap!r}")
 
     @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
@@ -56,3 +63,5 @@ class LinearHead(Part):
 
     def forward(self, ctx, x, logits) -> None:
         ctx.rt.kernels.gemm(x, self.weight, logits, STORE_F32)
+        if self.softcap is not None:
+            ctx.rt.kernels.softcap(logits, self.softcap)

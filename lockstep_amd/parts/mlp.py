@@ -89,3 +89,58 @@ class GatedMLP(FeedForward):
             return PendingAdd(partials)
         k.gemm(act, self.w_down, out, ADD_F32 if accumulate else STORE_F32)
         return None
+
+
+@register_part("clamped_gated_mlp")
+class ClampedGatedMLP(FeedForward):
+    """``down(g * sigmoid(alpha * g) * (u + 1))`` with ``g = min(gate(x), limit)`` and ``u = clamp(up(x),
+    -limit, limit)``: a gated unit whose two branches are bounded before they meet.  Parameters:
+    ``hidden_size``, ``intermediate_size``, ``limit``, ``alpha`` (the sigmoid's slope), and the tensor
+    names below the prefix ``gate_name``, ``up_name``, ``down_name``.
+
+    Gate and up are one matrix product over their rows one after the other, stored in float32; the
+    unit is a pass of its own in 32-bit that rounds to the compute dtype for the down product."""
+
+    graph_safe = True
+    repeatable = True
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        super().__init__(spec, prefix)
+        self.hidden = int(spec["hidden_size"])
+        self.inter = int(spec["intermediate_size"])
+        self.limit = float(spec["limit"])
+        self.alpha = float(spec["alpha"])
+        if not self.limit > 0:
+            raise ValueError(f"the gated unit's limit must be positive, got {self.limit}")
+        self.w_gate_up = self.w_down = None
+
+    @classmethod
+    def names(cls, spec: PartSpec, prefix: str):
+        p = spec.params
+        return tuple(f"{prefix}.{p.get(key, default)}" for key, default in
+                     (("gate_name", "gate"), ("up_name", "up"), ("down_name", "down")))
+
+    @classmethod
+    def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
+        h, i = int(spec["hidden_size"]), int(spec["intermediate_size"])
+        gate, up, down = cls.names(spec, prefix)
+        return [WeightSpec(gate, (i, h)), WeightSpec(up, (i, h)), WeightSpec(down, (h, i))]
+
+    def load(self, weights, rt) -> None:
+        gate_name, up_name, down_name = self.names(self.spec, self.prefix)
+        gate, up = weights.get(gate_name), weights.get(up_name)
+        if gate.dtype != up.dtype:
+            gate, up = gate.to(torch.float32), up.to(torch.float32)
+        self.w_gate_up = rt.matrix(torch.cat([gate, up], dim=0))
+        self.w_down = rt.matrix(weights.get(down_name))
+
+    def forward(self, ctx, x, out, accumulate: bool, defer: bool = False):
+        from .base import project_out
+
+        rt = ctx.rt
+        k = rt.kernels
+        wide = ctx.buf("mlp.gate_up", (ctx.n_tokens, 2 * self.inter), torch.float32)
+        k.gemm(x, self.w_gate_up, wide, STORE_F32)
+        act = ctx.buf("mlp.act", (ctx.n_tokens, self.inter), rt.dtype)
+        k.glu_clamped(wide, act, self.limit, self.alpha)
+        return project_out(ctx, act, self.w_down, out, accumulate, defer, "mlp.down_slices")

@@ -1,0 +1,154 @@
+"""Linear-attention mixers that keep a matrix of fixed size per request and head instead of keys
+and values: one recurrence with a decay and a write gate for every row of the state,
+
+    S_t = diag(a_t) S_(t-1) + b_t v_t^T          S [dim, vdim] in float32, zero at the start
+    o_t = S_t^T q_t
+
+of which HGRN2 and retention are two choices of (q, a, b):
+
+``hgrn2``      q = silu(W_q h); the forget gate f = lower + (1 - lower) * sigmoid(W_f h + bias) is both
+               the decay and, as 1 - f, what is written: a = f, b = 1 - f.  Each head's o is
+               RMS-normed over vdim with one weight for all heads, then W_o.
+``retention``  q = rotate(W_q h), b = rotate(W_k h) / sqrt(dim), a = the head's constant decay.  Each
+               head's o is divided by its root mean square (no weight), multiplied by
+               silu(W_g h), then W_o.
+
+The projections are one matrix product stored in float32; gates, rotation, the recurrence, the
+state and the per-head norm are computed in 32-bit.  The state lives in the cache manager's state
+slots: it is read at the start of a request's tokens of the step and left for the next step.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..config.base import PartSpec
+from ..ops import STORE_F32
+from .base import Mixer, StateSpec, WeightSpec, build_part, project_out, register_part
+
+
+class _LinearRecurrence(Mixer):
+    """What both mixers share: sizes, the state's declaration, the order of the launches."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        super().__init__(spec, prefix)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.heads, self.d, self.dv = int(p["num_heads"]), int(p["head_dim"]), int(p["value_dim"])
+        self.eps = float(p["eps"])
+        if min(self.heads, self.d, self.dv) <= 0:
+            raise ValueError("heads and sizes of a recurrent mixer must be positive")
+        self.w_in = self.w_o = None
+
+    def cache_spec(self):
+        return StateSpec((self.heads, self.d, self.dv), "float32")
+
+    def mixing_flops(self, tokens: int, start: int) -> float:
+        """Decay, write and read of every state element per token."""
+        return 5.0 * self.heads * self.d * self.dv * tokens
+
+    def _check_dim(self, rt) -> None:
+        most = rt.kernels.linrec_max_dim()
+        if self.d > most:
+            raise ValueError(f"a state of {self.d} rows a head is not supported: the recurrence kernel takes up to {most}")
+
+
+@register_part("hgrn2")
+class HGRN2(_LinearRecurrence):
+    """Parameters: ``hidden_size``, ``num_heads``, ``head_dim``, ``value_dim``, ``eps`` (of the per-head
+    norm).  Tensors below the prefix: ``q``, ``f`` ``[heads*dim, hidden]``, ``f.b``, ``lower``
+    ``[heads*dim]``, ``v`` ``[heads*vdim, hidden]``, ``norm`` ``[vdim]``, ``o`` ``[hidden, heads*vdim]``."""
+
+    @classmethod
+    def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
+        p = spec.params
+        h, n, d, dv = int(p["hidden_size"]), int(p["num_heads"]), int(p["head_dim"]), int(p["value_dim"])
+        return [WeightSpec(f"{prefix}.q", (n * d, h)), WeightSpec(f"{prefix}.f", (n * d, h)),
+                WeightSpec(f"{prefix}.f.b", (n * d,), kind="vector"), WeightSpec(f"{prefix}.lower", (n * d,), kind="vector"),
+                WeightSpec(f"{prefix}.v", (n * dv, h)), WeightSpec(f"{prefix}.norm", (dv,), kind="vector", init="norm"),
+                WeightSpec(f"{prefix}.o", (h, n * dv))]
+
+    def load(self, weights, rt) -> None:
+        self._check_dim(rt)
+        q, f, v = (weights.get(f"{self.prefix}.{n}") for n in "qfv")
+        if len({q.dtype, f.dtype, v.dtype}) > 1:
+            q, f, v = q.to(torch.float32), f.to(torch.float32), v.to(torch.float32)
+        self.w_in = rt.matrix(torch.cat([q, f, v], dim=0))
+        self.w_o = rt.matrix(weights.get(f"{self.prefix}.o"))
+        self.f_bias = rt.vector(weights.get(f"{self.prefix}.f.b"))
+        self.lower = rt.vector(weights.get(f"{self.prefix}.lower"))
+        self.norm = rt.vector(weights.get(f"{self.prefix}.norm"))
+        rt.kernels.mixers_lib()
+
+    def forward(self, ctx, run, x, out, accumulate: bool, defer: bool = False):
+        rt, k, t = ctx.rt, ctx.rt.kernels, ctx.n_tokens
+        n, d, dv = self.heads, self.d, self.dv
+        raw = ctx.buf("recurrence.in_f32", (t, 2 * n * d + n * dv), torch.float32)
+        k.gemm(x, self.w_in, raw, STORE_F32)
+        o = ctx.buf("recurrence.o_f32", (t, n * dv), torch.float32)
+        k.linrec(k.LINREC_HGRN2, raw, 0, n * d, 2 * n * d, n, d, dv, self.lower, self.f_bias, None, None, 0,
+                 ctx.max_position, ctx.seqs, ctx.n_seqs, ctx.cache.unit_state(run.cache), o)
+        normed = ctx.buf("recurrence.normed", (t, n * dv), rt.dtype)
+        k.head_norm_gate(o, n, dv, self.norm, None, self.eps, normed)
+        return project_out(ctx, normed, self.w_o, out, accumulate, defer, "recurrence.out_slices")
+
+
+@register_part("retention")
+class Retention(_LinearRecurrence):
+    """Parameters: ``hidden_size``, ``num_heads``, ``head_dim``, ``value_dim``, ``eps``, ``decay`` (one
+    number a head), ``position`` (a position-encoding ``PartSpec`` for q and k).  Tensors below the
+    prefix: ``q``, ``k`` ``[heads*dim, hidden]``, ``v``, ``g`` ``[heads*vdim, hidden]``, ``o``."""
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        super().__init__(spec, prefix)
+        self.decay = [float(v) for v in spec["decay"]]
+        if len(self.decay) != self.heads:
+            raise ValueError(f"{len(self.decay)} decays for {self.heads} heads")
+        self.position = build_part(spec["position"], prefix)
+        if self.position.rotary_dim > self.d:
+            raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head size {self.d}")
+
+    def parts(self):
+        return (self.position,)
+
+    @classmethod
+    def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
+        p = spec.params
+        h, n, d, dv = int(p["hidden_size"]), int(p["num_heads"]), int(p["head_dim"]), int(p["value_dim"])
+        return [WeightSpec(f"{prefix}.q", (n * d, h)), WeightSpec(f"{prefix}.k", (n * d, h)),
+                WeightSpec(f"{prefix}.v", (n * dv, h)), WeightSpec(f"{prefix}.g", (n * dv, h)),
+                WeightSpec(f"{prefix}.o", (h, n * dv))]
+
+    def load(self, weights, rt) -> None:
+        self._check_dim(rt)
+        tensors = [weights.get(f"{self.prefix}.{n}") for n in "qkvg"]
+        if len({t.dtype for t in tensors}) > 1:
+            tensors = [t.to(torch.float32) for t in tensors]
+        self.w_in = rt.matrix(torch.cat(tensors, dim=0))
+        self.w_o = rt.matrix(weights.get(f"{self.prefix}.o"))
+        self.decays = rt.vector(torch.tensor(self.decay, dtype=torch.float64))
+        rt.kernels.mixers_lib()
+        if hasattr(self.position, "bind"):
+            self.position.bind(rt)
+
+    def prepare_group(self):
+        share = getattr(self.position, "share_key", None)
+        return None if share is None else ("retention", share())
+
+    def prepare(self, ctx) -> None:
+        self.position.ensure(ctx.max_position + 1, ctx.rt)
+
+    def forward(self, ctx, run, x, out, accumulate: bool, defer: bool = False):
+        rt, k, t = ctx.rt, ctx.rt.kernels, ctx.n_tokens
+        n, d, dv = self.heads, self.d, self.dv
+        raw = ctx.buf("recurrence.in_f32", (t, 2 * n * d + 2 * n * dv), torch.float32)
+        k.gemm(x, self.w_in, raw, STORE_F32)
+        o = ctx.buf("recurrence.o_f32", (t, n * dv), torch.float32)
+        k.linrec(k.LINREC_RETENTION, raw, 0, n * d, 2 * n * d, n, d, dv, self.decays, None, self.position.cos,
+                 self.position.sin, self.position.rotary_dim, ctx.max_position, ctx.seqs, ctx.n_seqs,
+                 ctx.cache.unit_state(run.cache), o)
+        gated = ctx.buf("recurrence.normed", (t, n * dv), rt.dtype)
+        k.head_norm_gate(o, n, dv, None, raw[:, 2 * n * d + n * dv:], self.eps, gated)
+        return project_out(ctx, gated, self.w_o, out, accumulate, defer, "recurrence.out_slices")

@@ -1,0 +1,150 @@
+"""Attention whose heads exchange their scores before the softmax ("talking heads"), over the
+paged cache, with a sliding window that keeps the first tokens, keys and values of different
+sizes, biased projections, partial rotation and value mixing across layers.
+
+For the step's queries ``q_h`` (head h of H) and all cached keys ``k_g`` / values ``v_g`` (head g of
+G, query head h reads kv head ``h // (H/G)``):
+
+    raw_h[i, j] = scale * <q_h[i], k_kv(h)[j]>
+    s_h[i, j]   = sum_g talk[h, g] * raw_g[i, j]
+    j is visible to i  iff  j <= i and (i - j < window or j < keep_first)      (true positions)
+    o_h[i]      = sum_j softmax_j(s_h[i, :])[j] * v_kv(h)[j]
+
+Value mixing: the first layer of a model that mixes values keeps this step's values (``v_mix =
+"source"``); every later one (``v_mix = "mix"``) replaces its own by ``(1 - lambda) v + lambda
+v_first`` of the same token before they are cached, with its scalar ``lambda``.
+
+The projections are one matrix product over ``[Wq; Wk; Wv]`` stored in float32; one pass adds the
+biases, rotates, mixes values and writes queries, keys and values; one launch runs the attention
+of all requests of the step.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..config.base import PartSpec
+from ..ops import STORE_F32
+from .base import Mixer, PagedKVSpec, WeightSpec, build_part, project_out, register_part
+
+ROWS_A_BLOCK = 16      # query rows of a work item of the attention kernel
+
+
+@register_part("talking_attention")
+class TalkingAttention(Mixer):
+    """Parameters: ``hidden_size``, ``num_heads``, ``num_kv_heads``, ``head_dim`` (queries and keys),
+    ``value_dim``, ``position`` (a position-encoding ``PartSpec``), ``window``, ``keep_first``,
+    ``scale``, ``bias`` (biases of q, k, v), ``v_mix`` (None, ``"source"`` or ``"mix"``).  Tensors below
+    the prefix: ``q``, ``k``, ``v``, ``o``, ``talk`` ``[H, H]``, with ``bias`` also ``q.b``, ``k.b``,
+    ``v.b``, with ``v_mix`` also the scalar ``vmix`` (unused by the source layer)."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        super().__init__(spec, prefix)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.nq, self.nkv = int(p["num_heads"]), int(p["num_kv_heads"])
+        self.d, self.dv = int(p["head_dim"]), int(p["value_dim"])
+        self.window, self.keep_first = int(p["window"]), int(p.get("keep_first") or 0)
+        self.scale = float(p["scale"])
+        self.bias = bool(p.get("bias"))
+        self.v_mix = p.get("v_mix")
+        if self.nq % self.nkv:
+            raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} kv heads")
+        if self.window <= 0 or self.keep_first < 0:
+            raise ValueError(f"window {self.window} must be positive and keep_first {self.keep_first} not negative")
+        if self.v_mix not in (None, "source", "mix"):
+            raise ValueError(f"v_mix must be None, 'source' or 'mix', got {self.v_mix!r}")
+        self.position = build_part(p["position"], prefix)
+        if self.position.rotary_dim > self.d:
+            raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head size {self.d}")
+        self.w_qkv = self.w_o = self.b_qkv = self.talk = self.vmix = None
+
+    def parts(self):
+        return (self.position,)
+
+    @classmethod
+    def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
+        p = spec.params
+        h, nq, nkv = int(p["hidden_size"]), int(p["num_heads"]), int(p["num_kv_heads"])
+        d, dv = int(p["head_dim"]), int(p["value_dim"])
+        out = [WeightSpec(f"{prefix}.q", (nq * d, h)), WeightSpec(f"{prefix}.k", (nkv * d, h)),
+               WeightSpec(f"{prefix}.v", (nkv * dv, h)), WeightSpec(f"{prefix}.o", (h, nq * dv)),
+               WeightSpec(f"{prefix}.talk", (nq, nq), kind="vector")]
+        if p.get("bias"):
+            out += [WeightSpec(f"{prefix}.q.b", (nq * d,), kind="vector"), WeightSpec(f"{prefix}.k.b", (nkv * d,), kind="vector"),
+                    WeightSpec(f"{prefix}.v.b", (nkv * dv,), kind="vector")]
+        if p.get("v_mix"):
+            out.append(WeightSpec(f"{prefix}.vmix", (), kind="vector"))
+        return out
+
+    def cache_spec(self):
+        return PagedKVSpec(self.nkv, self.d, self.window, value_dim=self.dv, keep_first=self.keep_first)
+
+    def load(self, weights, rt) -> None:
+        q, k, v = (weights.get(f"{self.prefix}.{n}") for n in "qkv")
+        if len({q.dtype, k.dtype, v.dtype}) > 1:
+            q, k, v = q.to(torch.float32), k.to(torch.float32), v.to(torch.float32)
+        self.w_qkv = rt.matrix(torch.cat([q, k, v], dim=0))
+        self.w_o = rt.matrix(weights.get(f"{self.prefix}.o"))
+        self.talk = rt.vector(weights.get(f"{self.prefix}.talk"))
+        if self.bias:
+            self.b_qkv = rt.vector(torch.cat([weights.get(f"{self.prefix}.{n}.b").to(torch.float32) for n in "qkv"]))
+        if self.v_mix == "mix":
+            self.vmix = rt.vector(weights.get(f"{self.prefix}.vmix").reshape(1))
+        rt.kernels.mixers_lib()
+        rt.kernels.talking_lib(self.nq, self.nkv, self.d, self.dv)
+        if hasattr(self.position, "bind"):
+            self.position.bind(rt)
+
+    def mixing_flops(self, tokens: int, start: int) -> float:
+        """Scores, their mixing over the heads and value products over the (query, key) pairs a query sees."""
+        pairs = sum(min(start + i + 1, self.window + min(self.keep_first, max(0, start + i + 1 - self.window)))
+                    for i in range(tokens))
+        return (2.0 * self.d + 2.0 * self.dv + 2.0 * self.nq) * self.nq * pairs
+
+    def prepare_group(self):
+        share = getattr(self.position, "share_key", None)
+        return None if share is None else ("talking_attention", share())
+
+    def prepare(self, ctx) -> None:
+        self.position.ensure(ctx.max_position + 1, ctx.rt)
+        key = ("talking_attention", "blocks")
+        if ctx.declared(key):
+            return
+        # work items: (request of the step, block of its rows); single decoded tokens are one block each
+        if ctx.single_tokens:
+            pairs = np.stack([np.arange(ctx.n_seqs), np.zeros(ctx.n_seqs, dtype=np.int64)], axis=1)
+        else:
+            counts = -(-ctx.q_len // ROWS_A_BLOCK)
+            seq = np.repeat(np.arange(ctx.n_seqs), counts)
+            first = np.repeat(np.cumsum(counts) - counts, counts)
+            pairs = np.stack([seq, np.arange(int(counts.sum())) - first], axis=1)
+        ctx.declare(key, pairs.reshape(-1), signature=("talking_attention", len(pairs)))
+        ctx.notes[key] = len(pairs)
+
+    def forward(self, ctx, run, x, out, accumulate: bool, defer: bool = False):
+        rt = ctx.rt
+        k = rt.kernels
+        t = ctx.n_tokens
+        nq, nkv, d, dv = self.nq, self.nkv, self.d, self.dv
+        group, key_pages, value_pages = ctx.cache.unit_pages(run.cache)
+        if not run.writes_cache:
+            raise ValueError("a talking-heads attention layer writes its own keys and values")
+        raw = ctx.buf("talking.qkv_f32", (t, nq * d + nkv * (d + dv)), torch.float32)
+        k.gemm(x, self.w_qkv, raw, STORE_F32)
+        q = ctx.buf("talking.q", (t, nq * d), rt.dtype)
+        v_first = None
+        if self.v_mix is not None:
+            # this step's values of the first mixing layer: every token of the step, for the layers that follow
+            v_first = ctx.buf("talking.v_first", (t, nkv * dv), torch.float32)
+        k.talk_qkv(raw, t, nq, nkv, d, dv, self.b_qkv, self.position.cos, self.position.sin, self.position.rotary_dim,
+                   ctx.max_position, ctx.tok_seq, ctx.tok_pos, ctx.seqs, group.table, q, key_pages, value_pages,
+                   group.page_size, {None: 0, "source": 1, "mix": 2}[self.v_mix], self.vmix, v_first)
+        key = ("talking_attention", "blocks")
+        attn = ctx.buf("talking.out", (t, nq * dv), rt.dtype)
+        k.talk_attention(q, nq, nkv, d, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
+                         ctx.block(key), ctx.notes[key], self.talk, self.scale, self.window, self.keep_first, attn)
+        return project_out(ctx, attn, self.w_o, out, accumulate, defer, "talking.out_slices")
