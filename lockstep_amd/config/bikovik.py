@@ -120,9 +120,6 @@ class BikovikConfig(ModelConfig):
                                                     "mixer_norm_name": "norm1", "feed_forward_norm_name": "norm2"})
         mixing = [i for i, layer in enumerate(self.layers) if layer["type"] == "attention" and layer["mixer"].get("v_mix")]
         first_mixing = mixing[0] if mixing else None
-        shapes = {(self.layers[i]["mixer"]["kv_heads"], self.layers[i]["mixer"]["vdim"]) for i in mixing}
-        if len(shapes) > 1:
-            raise ConfigError(f"layers that mix values must agree on kv_heads and vdim, got {sorted(shapes)}")
         layers = []
         for i, layer in enumerate(self.layers):
             mlp = layer.get("mlp")
@@ -135,6 +132,9 @@ class BikovikConfig(ModelConfig):
                 prefix=f"l{i}", arrangement=arrangement, mixer=self._mixer(i, layer, first_mixing),
                 feed_forward=feed_forward, mixer_norm=norm,
                 feed_forward_norm=norm if mlp is not None else PartSpec("dynamic_tanh", {"size": width, "optional": True})))
+        shapes = {(layers[i].mixer["num_kv_heads"], layers[i].mixer["value_dim"]) for i in mixing}
+        if len(shapes) > 1:
+            raise ConfigError(f"layers that mix values must agree on kv_heads and vdim, got {sorted(shapes)}")
         return ModelSpec(
             hidden_size=width, vocab_size=self.vocab,
             embedding=PartSpec("token_embedding", {"name": "embed", "vocab_size": self.vocab, "hidden_size": width,

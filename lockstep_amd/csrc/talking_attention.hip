@@ -37,7 +37,7 @@ static_assert(H % G == 0, "query heads must be a multiple of the key/value heads
 static_assert(D % 8 == 0, "key size must be a multiple of 8");
 static_assert(DV % 4 == 0, "value size must be a multiple of 4");
 static_assert(H <= 32, "the heads' raw scores of a tile must fit into LDS");
-constexpr int NW = H % 4 == 0 ? 4 : (H % 2 == 0 ? 2 : 1);  // waves of a workgroup
+constexpr int NW = (H % 8 == 0 && H >= 32) ? 8 : (H % 4 == 0 ? 4 : (H % 2 == 0 ? 2 : 1));  // waves of a workgroup
 constexpr int HPW = H / NW;                                // heads a wave owns
 constexpr int VB = (DV + 15) / 16;                         // blocks of 16 value columns (the last may be partial)
 constexpr int kTileKeys = 32;

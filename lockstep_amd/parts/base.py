@@ -48,7 +48,8 @@ class WeightSpec:
     the compute dtype; ``vector`` tensors (norm weights, biases) are used in
     32-bit arithmetic and are kept in float32; ``int`` tensors are integer
     tables kept as int32.  ``init`` steers the random-weights mode: ``normal``
-    is N(0, std), ``norm`` is 1 + N(0, norm_std), ``zeros`` is 0.
+    is N(0, std), ``norm`` is 1 + N(0, norm_std), ``zeros`` is 0, ``identity`` is I + N(0, std) (a
+    square matrix), ``unit`` is uniform in (0, 1).
     """
 
     name: str

@@ -64,7 +64,7 @@ class DynamicTanh(Norm):
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
         name, size, optional = cls.tensor_name(spec, prefix), int(spec["size"]), bool(spec.params.get("optional"))
         return [WeightSpec(name, (size,), kind="vector", init="norm", optional=optional),
-                WeightSpec(f"{name}.b", (size,), kind="vector", init="zeros", optional=optional),
+                WeightSpec(f"{name}.b", (size,), kind="vector", optional=optional),
                 WeightSpec(f"{name}.alpha", (), kind="vector", init="norm", optional=optional)]
 
     def load(self, weights, rt) -> None:

@@ -66,7 +66,7 @@ class HGRN2(_LinearRecurrence):
         p = spec.params
         h, n, d, dv = int(p["hidden_size"]), int(p["num_heads"]), int(p["head_dim"]), int(p["value_dim"])
         return [WeightSpec(f"{prefix}.q", (n * d, h)), WeightSpec(f"{prefix}.f", (n * d, h)),
-                WeightSpec(f"{prefix}.f.b", (n * d,), kind="vector"), WeightSpec(f"{prefix}.lower", (n * d,), kind="vector"),
+                WeightSpec(f"{prefix}.f.b", (n * d,), kind="vector"), WeightSpec(f"{prefix}.lower", (n * d,), kind="vector", init="unit"),
                 WeightSpec(f"{prefix}.v", (n * dv, h)), WeightSpec(f"{prefix}.norm", (dv,), kind="vector", init="norm"),
                 WeightSpec(f"{prefix}.o", (h, n * dv))]
 

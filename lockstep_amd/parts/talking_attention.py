@@ -72,12 +72,12 @@ class TalkingAttention(Mixer):
         d, dv = int(p["head_dim"]), int(p["value_dim"])
         out = [WeightSpec(f"{prefix}.q", (nq * d, h)), WeightSpec(f"{prefix}.k", (nkv * d, h)),
                WeightSpec(f"{prefix}.v", (nkv * dv, h)), WeightSpec(f"{prefix}.o", (h, nq * dv)),
-               WeightSpec(f"{prefix}.talk", (nq, nq), kind="vector")]
+               WeightSpec(f"{prefix}.talk", (nq, nq), kind="vector", init="identity")]
         if p.get("bias"):
             out += [WeightSpec(f"{prefix}.q.b", (nq * d,), kind="vector"), WeightSpec(f"{prefix}.k.b", (nkv * d,), kind="vector"),
                     WeightSpec(f"{prefix}.v.b", (nkv * dv,), kind="vector")]
         if p.get("v_mix"):
-            out.append(WeightSpec(f"{prefix}.vmix", (), kind="vector"))
+            out.append(WeightSpec(f"{prefix}.vmix", (), kind="vector", init="unit"))
         return out
 
     def cache_spec(self):

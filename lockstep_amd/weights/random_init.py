@@ -3,7 +3,8 @@
 Each tensor gets its own generator seeded from ``(seed, tensor name)``, so a
 tensor's values do not depend on which other tensors the model has.  Matrices
 are N(0, std), norm weights are 1 + N(0, norm_std) (exactly 1 when norm_std is
-0); values are drawn in float32 and stored in ``dtype``.
+0), ``identity`` matrices are I + N(0, std), ``unit`` vectors are uniform in
+(0, 1); values are drawn in float32 and stored in ``dtype``.
 """
 
 from __future__ import annotations
@@ -45,6 +46,11 @@ def random_tensors(config: ModelConfig, seed: int, std: float | None = None, nor
                 value = value + torch.randn(w.shape, generator=gen, dtype=torch.float32) * norm_std
         elif w.init == "zeros":
             value = torch.zeros(w.shape, dtype=torch.float32)
+        elif w.init == "identity":
+            value = torch.eye(w.shape[0], w.shape[1], dtype=torch.float32)
+            value = value + torch.randn(w.shape, generator=gen, dtype=torch.float32) * std
+        elif w.init == "unit":
+            value = torch.rand(w.shape, generator=gen, dtype=torch.float32)
         else:
             value = torch.randn(w.shape, generator=gen, dtype=torch.float32) * std
         tensors[w.name] = value if w.kind == "int" else value.to(dtype)
