@@ -31,6 +31,14 @@ bench/throughput.py:35-45).  The value is all tokens (prompt and new) a second.
 
 measures a prompt in portions of 2,048 tokens and decode steps at batch 1, 8 and 64 at the
 context lengths of ``--contexts`` (default 4,096, 8,192 and 16,384 tokens).
+
+    python bench.py --workload designs [--model qwen3-0.6b] [--layers N]
+
+measures the Bikovik design (talking-heads attention over a window that keeps the first tokens,
+HGRN2 and retention layers, Dynamic Tanh norms, a clamped gated feed-forward) beside the Qwen3
+decoder at the same layer sizes (width, feed-forward, heads, head size, layers, vocabulary), both
+with random weights: prefill of one prompt and decode steps at batch 1 and 8, each with its
+fraction of the roofline.
 """
 
 from __future__ import annotations
@@ -115,7 +123,7 @@ def cache_bytes(spec, context: float, element: int) -> float:
     if spec is None:
         return 0.0
     if isinstance(spec, PagedKVSpec):
-        return min(context, spec.window or context) * 2 * spec.num_kv_heads * spec.head_dim * element
+        return min(context, spec.window or context) * spec.num_kv_heads * (spec.head_dim + spec.v_dim) * element
     if isinstance(spec, StateSpec):
         return _numel(spec.shape) * {"float32": 4, "int32": 4, "bfloat16": 2}[spec.dtype]
     raise TypeError(f"a cache unit described by {type(spec).__name__}: bench.py does not know its size")
@@ -323,11 +331,78 @@ def contexts_record(args, model, cfg, full_layers: int) -> dict:
     }
 
 
+def bikovik_like(qwen, layers: int, window: int = 4096, keep_first: int = 4):
+    """A Bikovik configuration at the layer sizes of the Qwen3 configuration ``qwen``: the layers cycle
+    through HGRN2, attention, retention, attention; every mixer has the heads and head size of the
+    Qwen3 attention (values as large as keys)."""
+    from lockstep_amd.config import config_from_dict
+
+    heads, kv, d = qwen.num_attention_heads, qwen.num_key_value_heads, qwen.head_dim
+    mlp = {"kind": "dense", "ff": qwen.intermediate_size, "limit": 7.0}
+    attention = {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "v_mix": True,
+        "mask": {"size": window, "keep_first": keep_first}, "rot": {"dims": d // 2, "base": qwen.rope_theta}}}
+    hgrn2 = {"type": "hgrn2", "mlp": mlp, "mixer": {"heads": heads, "dim": d, "vdim": d}}
+    retention = {"type": "retention", "mlp": mlp, "mixer": {
+        "heads": heads, "dim": d, "vdim": d, "rot": {"dims": d, "base": qwen.rope_theta},
+        "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, heads - 1)) for h in range(heads)]}}
+    cycle = [hgrn2, attention, retention, attention]
+    return config_from_dict({"architecture": "Bikovik", "vocab": qwen.vocab_size, "width": qwen.hidden_size,
+                             "embedding": {"scale": 1.0}, "norm": {"eps": qwen.rms_norm_eps}, "logit_softcap": 30.0,
+                             "layers": [cycle[i % 4] for i in range(layers)]})
+
+
+def designs_record(args) -> dict:
+    """Prefill and decode of the Bikovik design beside Qwen3 at equal layer sizes."""
+    import gc
+
+    import torch
+
+    from lockstep_amd.config.presets import preset
+    from lockstep_amd.engine.model import model_from_tensors
+    from lockstep_amd.weights import random_tensors
+
+    element = 2 if args.dtype == "bf16" else 4
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    qwen = preset(args.model, **({"num_hidden_layers": args.layers} if args.layers else {}))
+    layers = qwen.num_hidden_layers
+    out = {"workload": "designs", "sizes": args.model, "layers": layers, "dtype": args.dtype,
+           "prefill_tokens": args.prefill_len, "prompt_len": args.prompt_len, "steps": args.steps,
+           "data": "synthetic: uniform random token ids, random weights", "designs": {}}
+    for name, config in (("qwen3", qwen), ("bikovik", bikovik_like(qwen, layers))):
+        print(f"[bench] drawing random weights for {name} at {args.model} sizes", file=sys.stderr, flush=True)
+        tensors = random_tensors(config, seed=0, std=0.02, norm_std=0.0, dtype=torch.bfloat16)
+        model = model_from_tensors(config, tensors, dtype=dtype)
+        del tensors
+        work = Workload(model)
+        record = {}
+        seconds = measure_prefill(model, config, args.prefill_len, args.page_size, repeats=3)
+        flops = work.step_flops(args.prefill_len, 0, 1)
+        record["prefill"] = {"tok_s": round(args.prefill_len / seconds, 1), "ms": round(1e3 * seconds, 3),
+                             "frac_of_mfma_peak": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+        for batch in (1, 8):
+            times, context = measure_decode(model, config, batch, args.prompt_len, args.steps, args.warmup,
+                                            args.page_size, True, repeats=3)
+            elapsed = statistics.median(times)
+            moved = work.decode_bytes(batch, context, element)
+            record[f"decode_b{batch}"] = {"tok_s": round(batch * args.steps / elapsed, 1),
+                                          "ms_per_step": round(1e3 * elapsed / args.steps, 4),
+                                          "frac_of_hbm_peak": round(moved / (elapsed / args.steps) / PEAK_HBM, 4)}
+        record["kernels"] = kernel_digest(model)
+        out["designs"][name] = record
+        del model, work
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 def kernel_digest(model) -> str:
     """Names of the loaded kernel libraries; each carries a hash of its sources and flags, which
     fixes every tile and split constant (reference engine/kernels/registry.py:163-166)."""
     kernels = model.rt.kernels
     names = [Path(kernels.core_path).stem] + [Path(p).stem for _, p in sorted(kernels.attention_paths.items())]
+    names += [Path(kernels.mixers_path).stem] if kernels.mixers_path else []
+    names += [Path(p).stem for _, p in sorted(kernels.talking_paths.items())]
     return ",".join(n.replace("liblockstep_", "") for n in names)
 
 
@@ -458,9 +533,10 @@ def main(argv=None) -> int:
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     p.add_argument("--host-sampling", action="store_true",
                    help="pick every step's tokens on the host (Model.step + Sampler) instead of the device-side loop")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "reference-trace", "contexts"],
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "reference-trace", "contexts", "designs"],
                    help="decode: fixed batches (the headline); serve / reference-trace: a workload through the "
-                        "scheduler; contexts: prefill and decode at the context lengths of --contexts")
+                        "scheduler; contexts: prefill and decode at the context lengths of --contexts; designs: "
+                        "the Bikovik design beside Qwen3 at the layer sizes of --model")
     p.add_argument("--contexts", default="4096,8192,16384", help="contexts: the context lengths, comma separated")
     p.add_argument("--repeats", type=int, default=5, help="timed runs; the median is reported with the spread")
     p.add_argument("--requests", type=int, default=0, help="serve: only the first N requests of the workload")
@@ -479,6 +555,10 @@ def main(argv=None) -> int:
         return 2
 
     import torch
+
+    if args.workload == "designs":
+        print(json.dumps(designs_record(args)))
+        return 0
 
     model, cfg, full_layers = build_model(args)
     element = 2 if args.dtype == "bf16" else 4

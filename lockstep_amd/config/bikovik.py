@@ -47,6 +47,14 @@ class BikovikConfig(ModelConfig):
 
     architecture_names = ("Bikovik", "bikovik")
 
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
     @classmethod
     def from_dict(cls, raw) -> "BikovikConfig":
         # what the file does not mention does not exist: no soft cap, an embedding as stored

@@ -54,3 +54,16 @@ def test_init_writes_a_model_folder_from_a_preset_and_from_a_config(tmp_path):
 def test_run_needs_prompts_and_a_model():
     assert run("run", "--random", "tiny-a").returncode == 2          # no prompts
     assert run("run", "--prompt-ids", "1 2 3").returncode == 2       # neither --model nor --random
+
+
+def test_init_writes_a_bikovik_folder_from_its_preset(tmp_path):
+    from lockstep_amd.config import BikovikConfig, config_from_dir
+    from lockstep_amd.weights import SafetensorsFile
+
+    done = run("init", "--preset", "bikovik-tiny", "--out", str(tmp_path / "k"), "--seed", "2")
+    assert done.returncode == 0, done.stderr
+    config = config_from_dir(tmp_path / "k")
+    assert isinstance(config, BikovikConfig) and config.width == 128 and len(config.layers) == 4
+    names = SafetensorsFile(tmp_path / "k" / "model.safetensors").keys()
+    for name in ("embed", "head", "final.norm.alpha", "l0.mix.lower", "l1.mix.talk", "l3.mix.vmix", "l2.mix.g", "l2.mlp.down"):
+        assert name in names, name

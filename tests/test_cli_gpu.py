@@ -63,3 +63,22 @@ def test_run_random_weights_with_a_prompt_file(tmp_path):
     want = llm.generate([Request(uid=d["uid"], prompt=d["prompt"], seed=d["seed"], max_new_tokens=d["max_new_tokens"],
                                  temperature=d["temperature"], top_p=d["top_p"]) for d in lines])
     assert got == want and [len(got[f"q{i}"]) for i in range(4)] == [5, 6, 7, 8]
+
+
+def test_init_then_run_a_bikovik_folder(tmp_path):
+    """The same commands on the other architecture: the folder's config.json picks it."""
+    from lockstep_amd.weights.safetensors_io import open_model_tensors
+    from plain.bikovik_plain import PlainBikovik
+
+    folder = tmp_path / "k"
+    subprocess.run([*LOCKSTEP, "init", "--preset", "bikovik-tiny", "--out", str(folder), "--seed", "3", "--std", "0.2"],
+                   check=True, capture_output=True, timeout=300)
+    tensors = {name: handle.get(key) for name, (handle, key) in open_model_tensors(folder).items()}
+    plain = PlainBikovik(json.loads((folder / "config.json").read_text()), tensors)
+    prompts = [random_tokens(n, 512, seed=90 + n) for n in (3, 21, 70)]
+    want = {f"r{i:02d}": plain.generate_greedy(p, 6) for i, p in enumerate(prompts)}
+    args = [x for p in prompts for x in ("--prompt-ids", ",".join(map(str, p)))]
+    assert run("run", "--model", str(folder), "--dtype", "float32", "--max-new-tokens", "6", *args) == want
+    cut = run("run", "--model", str(folder), "--dtype", "float32", "--max-new-tokens", "6", "--prefill-chunk", "9",
+              "--max-batched-tokens", "20", "--block-size", "8", "--num-blocks", "40", "--decode-burst", "1", *args)
+    assert cut == want
