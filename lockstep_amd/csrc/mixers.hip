@@ -43,16 +43,23 @@ __global__ __launch_bounds__(256) void dyt_kernel(float* __restrict__ h, const f
   const long row = rows ? rows[r_out] : r_out;
   float* src = h + row * ldh;
   const float a = out ? alpha[0] : 0.f;
-  for (int e = threadIdx.x; e < width; e += 256) {
-    float v = src[e];
-    if (P) {
-      float sum = 0.f;
-      for (int s = 0; s < slices; ++s) sum = sum + P[s * p_stride + row * width + e];
-      v = v + sum;
-      src[e] = v;
+  // one element a thread (blockIdx.y walks the row): the slice sums of an element are requested together
+  const int e = blockIdx.y * 256 + threadIdx.x;
+  if (e >= width) return;
+  float v = src[e];
+  if (P) {
+    const float* p = P + row * width + e;
+    float sum = 0.f;
+    int s = 0;
+    for (; s + 4 <= slices; s += 4) {
+      const float p0 = p[s * p_stride], p1 = p[(s + 1) * p_stride], p2 = p[(s + 2) * p_stride], p3 = p[(s + 3) * p_stride];
+      sum = (((sum + p0) + p1) + p2) + p3;
     }
-    if (out) out[(long)r_out * ld_out + e] = from_f32<T>(tanhf(a * v) * weight[e] + bias[e]);
+    for (; s < slices; ++s) sum = sum + p[s * p_stride];
+    v = v + sum;
+    src[e] = v;
   }
+  if (out) out[(long)r_out * ld_out + e] = from_f32<T>(tanhf(a * v) * weight[e] + bias[e]);
 }
 
 // ---------------------------------------------------------------------------
@@ -153,106 +160,210 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 // mode 1 (retention): q = rotate(q_raw), b = rotate(k_raw) D^(-1/2), a = decay[head] for every row.
 // raw [T][ld] float holds q_raw at q_at, f_raw / k_raw at ab_at, v at v_at (H heads each).
 //
-// A workgroup takes (request, head, block of 64 columns of the state): wave g keeps the rows
-// [16 g, 16 g + 16) of its column in registers, one column a lane, and walks the request's tokens
-// in order, sixteen at a time: their q, a, b and v are prepared in LDS by all threads, every wave
-// adds its rows' part of o_t, and the parts are added in wave order.  The order of all sums is a
-// function of D alone.
+// Two launches.  The first computes q, a and b of every token once, elementwise over the whole step
+// (they do not depend on the state): gates [T][H][3][dp], dp = D rounded up to a multiple of 32,
+// zeros beyond D.  The second walks the tokens: a workgroup takes (request, head, block of 16
+// columns of the state).  A wave holds 32 rows of these columns: lane (column l16 = lane / 4,
+// quarter = lane % 4) keeps the rows 32 g + 8 quarter + {0..7} of its column in registers, and the
+// waves walk the request's tokens in order, sixteen at a time: their gates and values are copied to
+// LDS by all threads, every lane adds its rows' part of o_t (fused multiply-adds, written as
+// such), the four quarters of a column are neighbouring lanes and are added by exchanges inside the quad,
+// and the waves' parts are added in wave order.  The order of all sums is a function of D alone.
+//
+// The walk is software-pipelined over rounds of sixteen tokens, with two sets of LDS buffers: while
+// the waves walk the tokens of one round, the gates and values of the next are already requested
+// (into registers); after the walk they are written to the other set, one barrier follows, and the
+// waves' parts of the round's o_t are added and stored while the next round is walked.
 // ---------------------------------------------------------------------------
-constexpr int kRecRows = 16;    // rows of the state a lane keeps
-constexpr int kRecTokens = 16;  // tokens prepared at a time
+constexpr int kRecRows = 8;     // rows of the state a lane keeps
+constexpr int kRecCols = 16;    // columns of the state a workgroup takes
+constexpr int kRecWaveRows = 4 * kRecRows;  // rows a wave holds
+constexpr int kRecTokens = 16;  // tokens copied at a time
+constexpr int kRecPer = kRecTokens * 3 * kRecWaveRows / (4 * 64);  // vectors of four gates a thread copies a round
+constexpr int kRecVPer = kRecTokens * kRecCols / 64;                // the most values a thread fetches (one wave)
 
-__global__ __launch_bounds__(1024) void linrec_kernel(
-    int mode, const float* __restrict__ raw, long ld, int q_at, int ab_at, int v_at, int H, int D, int DV,
+__global__ __launch_bounds__(256) void linrec_gates_kernel(
+    int mode, const float* __restrict__ raw, long ld, int q_at, int ab_at, int n_tokens, int H, int D, int dp,
     const float* __restrict__ p0, const float* __restrict__ p1, const float* __restrict__ cos_table,
-    const float* __restrict__ sin_table, int rot, const SeqMeta* __restrict__ seqs, float* __restrict__ state,
-    float* __restrict__ out, long ldo) {
+    const float* __restrict__ sin_table, int rot, const int* __restrict__ tok_pos, float* __restrict__ gates) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)n_tokens * H * dp) return;
+  const int row = (int)(idx % dp), head = (int)((idx / dp) % H), t = (int)(idx / ((long)dp * H));
+  float q = 0.f, a = 0.f, b = 0.f;
+  if (row < D) {
+    const float* src = raw + (long)t * ld;
+    const int e = head * D + row;
+    if (mode == 0) {
+      const float lower = p0[e];
+      const float f = lower + (1.0f - lower) * sigmoidf_(src[ab_at + e] + (p1 ? p1[e] : 0.f));
+      q = siluf_(src[q_at + e]);
+      a = f;
+      b = 1.0f - f;
+    } else {
+      q = src[q_at + e];
+      b = src[ab_at + e];
+      if (row < rot) {
+        const int half = rot >> 1;
+        const int pe = row < half ? e + half : e - half;
+        const long pos = tok_pos[t];
+        q = rotate_element(q, src[q_at + pe], row, rot, cos_table + pos * half, sin_table + pos * half);
+        b = rotate_element(b, src[ab_at + pe], row, rot, cos_table + pos * half, sin_table + pos * half);
+      }
+      b = b * (1.0f / sqrtf((float)D));
+      a = p0[head];
+    }
+  }
+  float* dst = gates + ((long)t * H + head) * 3 * dp + row;
+  dst[0] = q;
+  dst[dp] = a;
+  dst[2 * dp] = b;
+}
+
+// Sum over the four neighbouring lanes 4k .. 4k + 3 (a DPP exchange inside the quad, no LDS traffic): first the
+// pairs (l, l ^ 1), then the pairs of pairs, so all four lanes end with the same bits.
+__device__ __forceinline__ float quad_sum(float v) {
+  v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));  // lanes 1 0 3 2
+  v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));  // lanes 2 3 0 1
+  return v;
+}
+
+__global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ gates, const float* __restrict__ raw,
+                                                     long ld, int v_at, int H, int D, int DV,
+                                                     const SeqMeta* __restrict__ seqs, float* __restrict__ state,
+                                                     float* __restrict__ out, long ldo) {
   extern __shared__ float lds[];
   const int seq = blockIdx.x / H, head = blockIdx.x % H, cb = blockIdx.y;
   const SeqMeta m = seqs[seq];
   if (m.q_len <= 0) return;
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6, waves = blockDim.x >> 6;
-  const int dp = waves * kRecRows;  // D rounded up to the rows the waves hold
-  float* q_s = lds;                                // [tokens][dp]
-  float* a_s = q_s + kRecTokens * dp;
-  float* b_s = a_s + kRecTokens * dp;
-  float* v_s = b_s + kRecTokens * dp;              // [tokens][64]
-  float* o_s = v_s + kRecTokens * 64;              // [waves][tokens][64]
-  const int c = cb * 64 + lane;
+  const int l16 = lane >> 2, quarter = lane & 3;  // four neighbouring lanes share a column
+  const int dp = waves * kRecWaveRows;  // D rounded up to the rows the waves hold
+  const int token = 3 * dp;             // floats of a token's gates: q, a, b
+  const int set = kRecTokens * token + kRecTokens * kRecCols + waves * kRecTokens * kRecCols;  // floats of one set
+  const int c = cb * kRecCols + l16;
   const bool col_ok = c < DV;
+  const int row0 = g * kRecWaveRows + quarter * kRecRows;
   float* mine = state + (((long)m.table_row * H + head) * D) * DV;
   float S[kRecRows];
 #pragma unroll
-  for (int r = 0; r < kRecRows; ++r) {
-    const int row = g * kRecRows + r;
-    S[r] = (row < D && col_ok) ? mine[(long)row * DV + c] : 0.f;
+  for (int r = 0; r < kRecRows; ++r) S[r] = (row0 + r < D && col_ok) ? mine[(long)(row0 + r) * DV + c] : 0.f;
+  const int v_per = (kRecTokens * kRecCols + (int)blockDim.x - 1) / (int)blockDim.x;
+  // a round's gates are kRecTokens * token consecutive floats of one head: token t at (t * H + head) * token.
+  // Thread i copies the vectors i, i + threads, ...; vector k lies in token k / (token / 4).
+  const int vec_a_token = token / 4;
+  int v_tt[kRecPer], v_in[kRecPer];
+#pragma unroll
+  for (int j = 0; j < kRecPer; ++j) {
+    const int k = j * (int)blockDim.x + (int)threadIdx.x;
+    v_tt[j] = k / vec_a_token;
+    v_in[j] = 4 * (k % vec_a_token);
   }
-  const float inv_sqrt_d = 1.0f / sqrtf((float)D);
-  const int half = rot >> 1;
-  for (int t0 = 0; t0 < m.q_len; t0 += kRecTokens) {
+  // the operands of the next round are requested before a round is walked
+  f32x4 rg[kRecPer];
+  float rv[kRecVPer];
+
+  auto request = [&](int t0) LS_INLINED {
     const int n = min(kRecTokens, m.q_len - t0);
-    for (int idx = threadIdx.x; idx < n * dp; idx += blockDim.x) {
-      const int tt = idx / dp, row = idx % dp;
-      float q = 0.f, a = 0.f, b = 0.f;
-      if (row < D) {
-        const float* src = raw + (long)(m.q_off + t0 + tt) * ld;
-        const int e = head * D + row;
-        if (mode == 0) {
-          const float lower = p0[e];
-          const float f = lower + (1.0f - lower) * sigmoidf_(src[ab_at + e] + (p1 ? p1[e] : 0.f));
-          q = siluf_(src[q_at + e]);
-          a = f;
-          b = 1.0f - f;
-        } else {
-          q = src[q_at + e];
-          b = src[ab_at + e];
-          if (row < rot) {
-            const int pe = row < half ? e + half : e - half;
-            const long pos = m.q_start + t0 + tt;
-            q = rotate_element(q, src[q_at + pe], row, rot, cos_table + pos * half, sin_table + pos * half);
-            b = rotate_element(b, src[ab_at + pe], row, rot, cos_table + pos * half, sin_table + pos * half);
-          }
-          b = b * inv_sqrt_d;
-          a = p0[head];
-        }
+#pragma unroll
+    for (int j = 0; j < kRecPer; ++j) {
+      const bool in = v_tt[j] < n;
+      const float* src = gates + ((long)(m.q_off + t0 + (in ? v_tt[j] : 0)) * H + head) * token + v_in[j];
+      rg[j] = *reinterpret_cast<const f32x4*>(src);
+    }
+#pragma unroll
+    for (int j = 0; j < kRecVPer; ++j) {
+      const int idx = j * (int)blockDim.x + (int)threadIdx.x;
+      const int tt = idx / kRecCols, col = cb * kRecCols + idx % kRecCols;
+      rv[j] = (j < v_per && tt < n && col < DV) ? raw[(long)(m.q_off + t0 + tt) * ld + v_at + head * DV + col] : 0.f;
+    }
+  };
+
+  auto deposit = [&](float* base) LS_INLINED {
+#pragma unroll
+    for (int j = 0; j < kRecPer; ++j)
+      *reinterpret_cast<f32x4*>(base + v_tt[j] * token + v_in[j]) = rg[j];
+    float* v_s = base + kRecTokens * token;  // [tokens][columns]
+#pragma unroll
+    for (int j = 0; j < kRecVPer; ++j) {
+      const int idx = j * (int)blockDim.x + (int)threadIdx.x;
+      if (j < v_per && idx < kRecTokens * kRecCols) v_s[idx] = rv[j];
+    }
+  };
+
+  // one round: walk the tokens of the set `base`, leave the waves' parts of o_t there
+  auto walk_round = [&](float* base, int n) LS_INLINED {
+    const float* v_s = base + kRecTokens * token;
+    float* o_s = base + kRecTokens * token + kRecTokens * kRecCols;  // [waves][tokens][columns]
+    // a token's operands: eight q, a and b of the lane's rows (two vectors each) and its column's value
+    struct Operands {
+      f32x4 q[2], a[2], b[2];
+      float v;
+    };
+    auto fetch = [&](int tt) LS_INLINED {
+      Operands x;
+      const float* qa = base + tt * token + row0;
+      x.v = v_s[tt * kRecCols + l16];
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        x.q[k] = *reinterpret_cast<const f32x4*>(qa + 4 * k);
+        x.a[k] = *reinterpret_cast<const f32x4*>(qa + dp + 4 * k);
+        x.b[k] = *reinterpret_cast<const f32x4*>(qa + 2 * dp + 4 * k);
       }
-      q_s[idx] = q;
-      a_s[idx] = a;
-      b_s[idx] = b;
-    }
-    for (int idx = threadIdx.x; idx < n * 64; idx += blockDim.x) {
-      const int tt = idx >> 6, col = cb * 64 + (idx & 63);
-      v_s[idx] = col < DV ? raw[(long)(m.q_off + t0 + tt) * ld + v_at + head * DV + col] : 0.f;
-    }
-    __syncthreads();
-    for (int tt = 0; tt < n; ++tt) {
-      const float v = v_s[tt * 64 + lane];
-      const float* qa = q_s + tt * dp + g * kRecRows;
-      const float* aa = a_s + tt * dp + g * kRecRows;
-      const float* ba = b_s + tt * dp + g * kRecRows;
+      return x;
+    };
+    auto step = [&](const Operands& x, int tt) LS_INLINED {
       float o = 0.f;
 #pragma unroll
       for (int r = 0; r < kRecRows; ++r) {
-        S[r] = aa[r] * S[r] + ba[r] * v;
-        o = o + S[r] * qa[r];
+        S[r] = fmaf(x.a[r >> 2][r & 3], S[r], x.b[r >> 2][r & 3] * x.v);
+        o = fmaf(S[r], x.q[r >> 2][r & 3], o);
       }
-      o_s[(g * kRecTokens + tt) * 64 + lane] = o;
+      o = quad_sum(o);  // the four quarters of the wave: rows 8 quarter .. of the same column
+      if (quarter == 0) o_s[(g * kRecTokens + tt) * kRecCols + l16] = o;
+    };
+    if (n == kRecTokens) {
+      // a full round is unrolled, and the operands of the token after next are requested before a token is walked
+      Operands ahead = fetch(0), next = fetch(1);
+#pragma unroll
+      for (int tt = 0; tt < kRecTokens; ++tt) {
+        const Operands now = ahead;
+        ahead = next;
+        if (tt + 2 < kRecTokens) next = fetch(tt + 2);
+        step(now, tt);
+      }
+    } else {
+      for (int tt = 0; tt < n; ++tt) step(fetch(tt), tt);
     }
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < n * 64; idx += blockDim.x) {
-      const int tt = idx >> 6, l = idx & 63, col = cb * 64 + l;
+  };
+
+  // the waves' parts of a round are added in wave order and stored (while the next round is walked: that round
+  // writes the other set, and the barrier at its end stands before the round after it writes this one again)
+  auto store_round = [&](const float* base, int t0, int n) LS_INLINED {
+    const float* o_s = base + kRecTokens * token + kRecTokens * kRecCols;
+    for (int idx = threadIdx.x; idx < n * kRecCols; idx += blockDim.x) {
+      const int tt = idx / kRecCols, l = idx % kRecCols, col = cb * kRecCols + l;
       float o = 0.f;
-      for (int w = 0; w < waves; ++w) o = o + o_s[(w * kRecTokens + tt) * 64 + l];
+      for (int w = 0; w < waves; ++w) o = o + o_s[(w * kRecTokens + tt) * kRecCols + l];
       if (col < DV) out[(long)(m.q_off + t0 + tt) * ldo + head * DV + col] = o;
     }
-    // (the next round's preparation writes q_s .. v_s only, which no thread reads any more; its
-    // barrier stands between these reads of o_s and the next writes to it)
+  };
+
+  request(0);
+  deposit(lds);
+  __syncthreads();
+  int at = 0;
+  for (int t0 = 0; t0 < m.q_len; t0 += kRecTokens, at ^= 1) {
+    const int n = min(kRecTokens, m.q_len - t0);
+    const bool more = t0 + kRecTokens < m.q_len;
+    if (more) request(t0 + kRecTokens);
+    walk_round(lds + at * set, n);
+    if (more) deposit(lds + (at ^ 1) * set);
+    __syncthreads();
+    store_round(lds + at * set, t0, n);
   }
 #pragma unroll
-  for (int r = 0; r < kRecRows; ++r) {
-    const int row = g * kRecRows + r;
-    if (row < D && col_ok) mine[(long)row * DV + c] = S[r];
-  }
+  for (int r = 0; r < kRecRows; ++r)
+    if (row0 + r < D && col_ok) mine[(long)(row0 + r) * DV + c] = S[r];
 }
 
 // ---------------------------------------------------------------------------
@@ -300,10 +411,10 @@ extern "C" int ls_dyt(int dtype, float* h, const float* P, int slices, int p_row
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const long p_stride = (long)p_rows * width;
   if (dtype == kF32)
-    hipLaunchKernelGGL(dyt_kernel<float>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_stride, weight, bias, alpha,
+    hipLaunchKernelGGL(dyt_kernel<float>, dim3(n_rows, (width + 255) / 256), dim3(256), 0, s, h, P, slices, p_stride, weight, bias, alpha,
                        (float*)out, rows, width, ldh, ld_out);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(dyt_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_stride, weight, bias, alpha,
+    hipLaunchKernelGGL(dyt_kernel<bf16_t>, dim3(n_rows, (width + 255) / 256), dim3(256), 0, s, h, P, slices, p_stride, weight, bias, alpha,
                        (bf16_t*)out, rows, width, ldh, ld_out);
   else
     return fail("dyt: unknown dtype %d", dtype);
@@ -367,27 +478,34 @@ extern "C" int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, i
   return check_launch("talk_qkv");
 }
 
-extern "C" int ls_linrec_max_dim() { return 64 * kRecRows / 4; }
+extern "C" int ls_linrec_max_dim() { return 8 * kRecWaveRows; }
 
-extern "C" int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_at, int v_at, int H, int D, int DV,
-                         const float* p0, const float* p1, const float* cos_table, const float* sin_table, int rot,
-                         int table_positions, int max_pos, const void* seqs, int n_seqs, float* state, float* out,
-                         long ldo, void* stream) {
+extern "C" long ls_linrec_gate_floats(int n_tokens, int H, int D) {
+  const int dp = (D + kRecWaveRows - 1) / kRecWaveRows * kRecWaveRows;
+  return (long)n_tokens * H * 3 * dp;
+}
+
+extern "C" int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_at, int v_at, int n_tokens, int H, int D,
+                         int DV, const float* p0, const float* p1, const float* cos_table, const float* sin_table,
+                         int rot, int table_positions, int max_pos, const int* tok_pos, const void* seqs, int n_seqs,
+                         float* state, float* gates, float* out, long ldo, void* stream) {
   LS_REQUIRE(mode == 0 || mode == 1, "linrec: unknown mode %d", mode);
-  LS_REQUIRE(n_seqs > 0 && H > 0 && D > 0 && DV > 0 && D <= ls_linrec_max_dim(),
+  LS_REQUIRE(n_seqs > 0 && n_tokens > 0 && H > 0 && D > 0 && DV > 0 && D <= ls_linrec_max_dim(),
              "linrec: bad sizes (heads %d, rows %d of at most %d, columns %d)", H, D, ls_linrec_max_dim(), DV);
-  LS_REQUIRE(raw && seqs && state && out && p0 && ldo >= (long)H * DV, "linrec: bad operands");
+  LS_REQUIRE(raw && seqs && state && out && p0 && gates && ldo >= (long)H * DV, "linrec: bad operands");
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(gates) % 16 == 0, "linrec: the gates must be 16-byte aligned");
   LS_REQUIRE(q_at >= 0 && ab_at >= 0 && v_at >= 0 && ld >= q_at + (long)H * D && ld >= ab_at + (long)H * D &&
                  ld >= v_at + (long)H * DV,
              "linrec: the projections do not fit the rows");
   if (mode == 1) {
     LS_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "linrec: %d rotated dimensions of %d", rot, D);
-    LS_REQUIRE(rot == 0 || (cos_table && sin_table && max_pos < table_positions),
+    LS_REQUIRE(rot == 0 || (cos_table && sin_table && tok_pos && max_pos < table_positions),
                "linrec: position %d is beyond the rotation tables (%d)", max_pos, table_positions);
   }
-  const int waves = (D + kRecRows - 1) / kRecRows;
-  const int dp = waves * kRecRows;
-  const size_t lds = sizeof(float) * (size_t)(3 * kRecTokens * dp + kRecTokens * 64 + waves * kRecTokens * 64);
+  const int waves = (D + kRecWaveRows - 1) / kRecWaveRows;
+  const int dp = waves * kRecWaveRows;
+  const size_t lds =
+      2 * sizeof(float) * (size_t)(3 * kRecTokens * dp + kRecTokens * kRecCols + waves * kRecTokens * kRecCols);
   if (lds > 48 * 1024) {  // (more than the default bound of dynamic LDS: say so once a size)
     static size_t allowed = 0;
     if (lds > allowed) {
@@ -397,9 +515,12 @@ extern "C" int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_a
       allowed = lds;
     }
   }
-  dim3 grid((unsigned)(n_seqs * H), (unsigned)((DV + 63) / 64));
-  hipLaunchKernelGGL(linrec_kernel, grid, dim3(64 * waves), lds, reinterpret_cast<hipStream_t>(stream), mode, raw, ld,
-                     q_at, ab_at, v_at, H, D, DV, p0, p1, cos_table, sin_table, mode == 1 ? rot : 0,
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const long elements = (long)n_tokens * H * dp;
+  hipLaunchKernelGGL(linrec_gates_kernel, dim3((unsigned)((elements + 255) / 256)), dim3(256), 0, s, mode, raw, ld, q_at,
+                     ab_at, n_tokens, H, D, dp, p0, p1, cos_table, sin_table, mode == 1 ? rot : 0, tok_pos, gates);
+  dim3 grid((unsigned)(n_seqs * H), (unsigned)((DV + kRecCols - 1) / kRecCols));
+  hipLaunchKernelGGL(linrec_kernel, grid, dim3(64 * waves), lds, s, gates, raw, ld, v_at, H, D, DV,
                      (const SeqMeta*)seqs, state, out, ldo);
   return check_launch("linrec");
 }

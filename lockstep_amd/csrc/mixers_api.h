@@ -32,11 +32,14 @@ int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, int H, int G
 
 // Linear recurrence S_t = diag(a_t) S_(t-1) + b_t v_t^T, o_t = S_t^T q_t over the tokens of every request of the
 // step, state [slots][H][D][DV] float (mode 0: HGRN2 gates from p0 = lower bounds [H*D] and p1 = gate bias or null;
-// mode 1: retention with p0 = decay [H] and rotated q, k).  out [T][ldo] float gets o_t.
+// mode 1: retention with p0 = decay [H] and rotated q, k at the positions tok_pos [n_tokens]).  out [T][ldo] float
+// gets o_t.  gates: scratch of ls_linrec_gate_floats(n_tokens, H, D) floats, 16-byte aligned.
 int ls_linrec_max_dim();
-int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_at, int v_at, int H, int D, int DV, const float* p0,
-              const float* p1, const float* cos_table, const float* sin_table, int rot, int table_positions,
-              int max_pos, const void* seqs, int n_seqs, float* state, float* out, long ldo, void* stream);
+long ls_linrec_gate_floats(int n_tokens, int H, int D);
+int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_at, int v_at, int n_tokens, int H, int D, int DV,
+              const float* p0, const float* p1, const float* cos_table, const float* sin_table, int rot,
+              int table_positions, int max_pos, const int* tok_pos, const void* seqs, int n_seqs, float* state,
+              float* gates, float* out, long ldo, void* stream);
 
 // Per (token, head): x [DV] / sqrt(mean(x^2) + eps), times weight [DV] and silu(gate) where given.
 int ls_head_norm_gate(int out_dtype, const float* x, long ldx, int n_tokens, int H, int DV, const float* weight,

@@ -20,6 +20,10 @@
 //      (row statistics over the four lanes that share a query row);
 //   3. O^T += V^T P^T per head with the atom (value columns are the first operand, so the lane
 //      that holds a row's statistics also holds the row's accumulators).
+// A step of single decoded tokens has one row block a request, which would leave most of the GPU
+// idle while one workgroup walks the whole window: there a request's tiles are dealt to several work
+// items in contiguous runs, each leaves (max, sum, unnormalised output) of its run for the request's
+// one row, and a second kernel folds the runs in ascending order.
 // Scores, weights, statistics and accumulators are float; products read the compute dtype T.
 // Keys a request does not hold (beyond its length, pages a window has released) enter as zeros and
 // are masked; their values are replaced by zeros before the product.
@@ -37,10 +41,13 @@ static_assert(H % G == 0, "query heads must be a multiple of the key/value heads
 static_assert(D % 8 == 0, "key size must be a multiple of 8");
 static_assert(DV % 4 == 0, "value size must be a multiple of 4");
 static_assert(H <= 32, "the heads' raw scores of a tile must fit into LDS");
-constexpr int NW = (H % 8 == 0 && H >= 32) ? 8 : (H % 4 == 0 ? 4 : (H % 2 == 0 ? 2 : 1));  // waves of a workgroup
+constexpr int NW = H % 8 == 0 ? 8 : (H % 4 == 0 ? 4 : (H % 2 == 0 ? 2 : 1));  // waves of a workgroup
 constexpr int HPW = H / NW;                                // heads a wave owns
 constexpr int VB = (DV + 15) / 16;                         // blocks of 16 value columns (the last may be partial)
 constexpr int kTileKeys = 32;
+constexpr int GS = H / G;  // query heads that read one key/value head
+// consecutive own heads of a wave that read the same key/value head: its keys and values are loaded once for them
+constexpr int SH = HPW % GS == 0 ? GS : (GS % HPW == 0 ? HPW : 1);
 
 struct SeqMeta {
   int q_off, q_len, q_start, kv_len, table_row, reserved[3];
@@ -58,12 +65,15 @@ template <typename T>
 __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
     const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ blocks,
-    const float* __restrict__ talk, float scale, int window, int keep_first, T* __restrict__ out, long ldo) {
+    const float* __restrict__ talk, float scale, int window, int keep_first, T* __restrict__ out, long ldo,
+    float* __restrict__ part) {
   constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
   constexpr int KCH = (D + KC - 1) / KC;  // chunks of a key (lanes beyond D in the last one bring zeros)
-  __shared__ float raw_s[H][2][4][64];  // [head][half of the tile][i][lane]
+  __shared__ f32x4 raw_s[H][2][64];  // [head][half of the tile][lane]: the lane's four keys of that half
   __shared__ float talk_s[H * H];
-  const int seq = blocks[2 * blockIdx.x], rb = blocks[2 * blockIdx.x + 1];
+  // a work item: request of the step, block of 16 of its rows, which run of the tiles, of how many runs
+  const int seq = blocks[4 * blockIdx.x], rb = blocks[4 * blockIdx.x + 1];
+  const int run = blocks[4 * blockIdx.x + 2], n_runs = max(1, blocks[4 * blockIdx.x + 3]);
   const SeqMeta m = seqs[seq];
   const int row0 = rb * 16;
   if (row0 >= m.q_len) return;
@@ -93,33 +103,54 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
   const int n_tiles = kept_tiles + (hi_tile - lo_tile + 1);
   __syncthreads();
 
-  for (int step = 0; step < n_tiles; ++step) {
+  const int per_run = (n_tiles + n_runs - 1) / n_runs;
+  const int step_end = min(n_tiles, (run + 1) * per_run);
+  for (int step = run * per_run; step < step_end; ++step) {
     const int tile = step < kept_tiles ? step : lo_tile + (step - kept_tiles);
     const int key0 = tile * kTileKeys;
     // -- 1. transposed raw scores of the wave's own heads ------------------------------------
+    // page and slot of the lane's key of each half (as a row of K), and of its four keys (as columns of V^T)
+    long k_at[2], v_at[2];
+    bool k_ok[2], v_ok[2][4];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int key = key0 + 16 * half + l16;
       const int page = key <= p_last ? my_table[key / page_size] : -1;
-      const bool key_ok = page >= 0;
-      const long slot_at = ((long)(key_ok ? page : 0) * G) * page_size + (key_ok ? key % page_size : 0);
+      k_ok[half] = page >= 0;
+      k_at[half] = ((long)(page >= 0 ? page : 0) * G) * page_size + (page >= 0 ? key % page_size : 0);
+      const int key4 = key0 + 16 * half + 4 * quad;
+      const int page4 = key4 <= p_last ? my_table[key4 / page_size] : -1;
+      v_at[half] = ((long)(page4 >= 0 ? page4 : 0) * G * DV) * page_size + (page4 >= 0 ? key4 % page_size : 0);
 #pragma unroll
-      for (int x = 0; x < HPW; ++x) {
-        const int h = w * HPW + x, g = h / (H / G);
-        const T* k_row = k_pages + (slot_at + (long)g * page_size) * D;
-        f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < 4; ++i) v_ok[half][i] = page4 >= 0 && key4 + i <= p_last;
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+      for (int xg = 0; xg < HPW / SH; ++xg) {
+        const int g = (w * HPW + xg * SH) / GS;
+        const T* k_row = k_pages + (k_at[half] + (long)g * page_size) * D;
+        typename Atom<T>::vec_t kv[KCH];
 #pragma unroll
         for (int c = 0; c < KCH; ++c) {
           const bool in = c * KC + VEC * quad + VEC <= D;
-          const int at = in ? c * KC + VEC * quad : 0;
-          Atom<T>::mma(s, load_or_zero<T>(k_row + at, key_ok && in), load_or_zero<T>(q_row + h * D + at, row_ok && in));
+          kv[c] = load_or_zero<T>(k_row + (in ? c * KC + VEC * quad : 0), k_ok[half] && in);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) raw_s[h][half][i][lane] = s[i] * scale;
+        for (int xs = 0; xs < SH; ++xs) {
+          const int h = w * HPW + xg * SH + xs;
+          f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < KCH; ++c) {
+            const bool in = c * KC + VEC * quad + VEC <= D;
+            Atom<T>::mma(s, kv[c], load_or_zero<T>(q_row + h * D + (in ? c * KC + VEC * quad : 0), row_ok && in));
+          }
+          raw_s[h][half][lane] = f32x4{s[0] * scale, s[1] * scale, s[2] * scale, s[3] * scale};
+        }
       }
     }
     __syncthreads();
-    // -- 2. mix, mask, online softmax; 3. values ------------------------------------------------
+    // -- 2. mix, mask, online softmax ---------------------------------------------------------------
     bool see[2][4];
 #pragma unroll
     for (int half = 0; half < 2; ++half)
@@ -128,80 +159,99 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
         const int key = key0 + 16 * half + 4 * quad + i;
         see[half][i] = row_ok && key <= my_pos && (my_pos - key < window || key < keep_first);
       }
+    // every head's raw scores are read once and go into all of the wave's own heads
+    float mixed[HPW][2][4];
 #pragma unroll
-    for (int x = 0; x < HPW; ++x) {
-      const int h = w * HPW + x, g = h / (H / G);
-      float s[2][4];
+    for (int x = 0; x < HPW; ++x)
 #pragma unroll
       for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s[half][i] = 0.f;
-      for (int o = 0; o < H; ++o) {
-        const float weight = talk_s[h * H + o];
+        for (int i = 0; i < 4; ++i) mixed[x][half][i] = 0.f;
 #pragma unroll
-        for (int half = 0; half < 2; ++half)
+    for (int o = 0; o < H; ++o) {
+      const f32x4 r0 = raw_s[o][0][lane], r1 = raw_s[o][1][lane];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) s[half][i] = s[half][i] + weight * raw_s[o][half][i][lane];
+      for (int x = 0; x < HPW; ++x) {
+        const float weight = talk_s[(w * HPW + x) * H + o];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          mixed[x][0][i] = mixed[x][0][i] + weight * r0[i];
+          mixed[x][1][i] = mixed[x][1][i] + weight * r1[i];
+        }
       }
+    }
+    float shrink[HPW];
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) {     // the scores become the weights, in place
       float top = kNegSentinel;
 #pragma unroll
       for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) top = fmaxf(top, see[half][i] ? s[half][i] : kNegSentinel);
+        for (int i = 0; i < 4; ++i) top = fmaxf(top, see[half][i] ? mixed[x][half][i] : kNegSentinel);
       top = quad16_max(top);
       const float m_new = fmaxf(m_run[x], top);
-      const float shrink = softmax_exp<T>(m_run[x] - m_new);
-      float p[2][4], sum = 0.f;
+      shrink[x] = softmax_exp<T>(m_run[x] - m_new);
+      float sum = 0.f;
 #pragma unroll
       for (int half = 0; half < 2; ++half)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          p[half][i] = see[half][i] ? softmax_exp<T>(s[half][i] - m_new) : 0.f;
-          sum = sum + p[half][i];
+          mixed[x][half][i] = see[half][i] ? softmax_exp<T>(mixed[x][half][i] - m_new) : 0.f;
+          sum = sum + mixed[x][half][i];
         }
       sum = quad16_sum(sum);
-      l_run[x] = l_run[x] * shrink + sum;
+      l_run[x] = l_run[x] * shrink[x] + sum;
       m_run[x] = m_new;
-      // values of the tile's keys, value column 16 b + l16, keys 4 quad .. 4 quad + 3 of each half
-      long v_at[2];
-      bool v_ok[2][4];
+    }
+    // -- 3. values: column 16 b + l16 of V^T, keys 4 quad .. 4 quad + 3 of each half ----------------
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int key = key0 + 16 * half + 4 * quad;
-        const int page = key <= p_last ? my_table[key / page_size] : -1;
-        v_at[half] = (((long)(page >= 0 ? page : 0) * G + g) * DV) * page_size + (page >= 0 ? key % page_size : 0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v_ok[half][i] = page >= 0 && key + i <= p_last;
-      }
+    for (int xg = 0; xg < HPW / SH; ++xg) {
+      const int g = (w * HPW + xg * SH) / GS;
 #pragma unroll
       for (int b = 0; b < VB; ++b) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[x][b][i] = acc[x][b][i] * shrink;
         const bool col_ok = 16 * b + l16 < DV;
-        const long column = (long)(col_ok ? 16 * b + l16 : 0) * page_size;
+        const long column = ((long)g * DV + (col_ok ? 16 * b + l16 : 0)) * page_size;
         if constexpr (sizeof(T) == 2) {
           const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[0] + column);
           const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[1] + column);
-          bf16x8 a, pb;
+          bf16x8 a;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             a[i] = (v_ok[0][i] && col_ok) ? v0[i] : (bf16_t)0.f;
             a[4 + i] = (v_ok[1][i] && col_ok) ? v1[i] : (bf16_t)0.f;
-            pb[i] = (bf16_t)p[0][i];
-            pb[4 + i] = (bf16_t)p[1][i];
           }
-          Atom<T>::mma(acc[x][b], a, pb);
+#pragma unroll
+          for (int xs = 0; xs < SH; ++xs) {
+            const int x = xg * SH + xs;
+            bf16x8 pb;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              acc[x][b][i] = acc[x][b][i] * shrink[x];
+              pb[i] = (bf16_t)mixed[x][0][i];
+              pb[4 + i] = (bf16_t)mixed[x][1][i];
+            }
+            Atom<T>::mma(acc[x][b], a, pb);
+          }
         } else {
+          f32x4 a[2];
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             const f32x4 v = *reinterpret_cast<const f32x4*>(v_pages + v_at[half] + column);
-            f32x4 a, pb;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              a[i] = (v_ok[half][i] && col_ok) ? v[i] : 0.f;
-              pb[i] = p[half][i];
+            for (int i = 0; i < 4; ++i) a[half][i] = (v_ok[half][i] && col_ok) ? v[i] : 0.f;
+          }
+#pragma unroll
+          for (int xs = 0; xs < SH; ++xs) {
+            const int x = xg * SH + xs;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[x][b][i] = acc[x][b][i] * shrink[x];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+              f32x4 pb;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) pb[i] = mixed[x][half][i];
+              Atom<T>::mma(acc[x][b], a[half], pb);
             }
-            Atom<T>::mma(acc[x][b], a, pb);
           }
         }
       }
@@ -209,6 +259,24 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
     __syncthreads();
   }
   if (!row_ok) return;
+  if (n_runs > 1) {
+    // (single decoded tokens: row 0 only) [item][head][DV + 2]: the unnormalised output, then max and sum
+    if (l16 != 0) return;
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) {
+      float* dst = part + ((long)blockIdx.x * H + w * HPW + x) * (DV + 2);
+#pragma unroll
+      for (int b = 0; b < VB; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (16 * b + 4 * quad + i < DV) dst[16 * b + 4 * quad + i] = acc[x][b][i];
+      if (quad == 0) {
+        dst[DV] = m_run[x];
+        dst[DV + 1] = l_run[x];
+      }
+    }
+    return;
+  }
   T* dst = out + (long)(m.q_off + row0 + l16) * ldo;
 #pragma unroll
   for (int x = 0; x < HPW; ++x) {
@@ -219,6 +287,29 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         if (16 * b + 4 * quad + i < DV) dst[h * DV + 16 * b + 4 * quad + i] = from_f32<T>(acc[x][b][i] * inv);
+  }
+}
+
+// Fold the runs of a decoded token: for request `seq` (one row) and head h, the partial results of the
+// items seq * n_runs .. seq * n_runs + n_runs - 1 in ascending order.  One workgroup a (request, head).
+template <typename T>
+__global__ __launch_bounds__(64) void talk_combine_kernel(const float* __restrict__ part, int n_runs,
+                                                          const SeqMeta* __restrict__ seqs, T* __restrict__ out,
+                                                          long ldo) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const SeqMeta m = seqs[seq];
+  if (m.q_len <= 0) return;
+  const float* mine = part + ((long)seq * n_runs * H + h) * (DV + 2);
+  const long stride = (long)H * (DV + 2);
+  float top = kNegSentinel;
+  for (int r = 0; r < n_runs; ++r) top = fmaxf(top, mine[r * stride + DV]);
+  float total = 0.f;
+  for (int r = 0; r < n_runs; ++r) total = total + mine[r * stride + DV + 1] * softmax_exp<T>(mine[r * stride + DV] - top);
+  const float inv = 1.0f / total;
+  for (int c = threadIdx.x; c < DV; c += 64) {
+    float sum = 0.f;
+    for (int r = 0; r < n_runs; ++r) sum = sum + mine[r * stride + c] * softmax_exp<T>(mine[r * stride + DV] - top);
+    out[(long)m.q_off * ldo + h * DV + c] = from_f32<T>(sum * inv);
   }
 }
 
@@ -234,12 +325,16 @@ extern "C" int ls_talk_dim() { return D; }
 extern "C" int ls_talk_vdim() { return DV; }
 
 // q [T][ldq] (rotated queries, H heads of D); key pages [pages][G][page_size][D], value pages
-// [pages][G][DV][page_size]; table [slots][table_stride]; seqs: the step's requests; blocks: n_blocks pairs
-// (request of the step, block of 16 of its rows); talk [H][H] float; out [T][ldo] (H heads of DV).
+// [pages][G][DV][page_size]; table [slots][table_stride]; seqs: the step's requests; blocks: n_blocks work items
+// of four ints (request of the step, block of 16 of its rows, run, runs); talk [H][H] float; out [T][ldo] (H heads
+// of DV).  n_runs > 1: a step of single decoded tokens whose request i has the items i * n_runs .. (one a run);
+// part then holds n_blocks * H * (DV + 2) floats, and a second launch folds the runs into out.
 extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages,
                                  int page_size, const int* table, int table_stride, const void* seqs,
                                  const int* blocks, int n_blocks, const float* talk, float scale, int window,
-                                 int keep_first, void* out, long ldo, void* stream) {
+                                 int keep_first, void* out, long ldo, int n_runs, float* part, void* stream) {
+  LS_REQUIRE(n_runs >= 1 && (n_runs == 1 || (part && n_blocks % n_runs == 0)), "talk_attention: %d runs over %d items",
+             n_runs, n_blocks);
   LS_REQUIRE(n_blocks > 0 && q && k_pages && v_pages && table && seqs && blocks && talk && out, "talk_attention: null operand");
   LS_REQUIRE(ldq >= (long)H * D && ldo >= (long)H * DV, "talk_attention: rows are too short");
   LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && table_stride > 0, "talk_attention: page size %d", page_size);
@@ -252,12 +347,18 @@ extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void*
     LS_REQUIRE(ldq % 4 == 0, "talk_attention: query rows must be 16-byte aligned");
     hipLaunchKernelGGL(talk_attention_kernel<float>, dim3(n_blocks), dim3(64 * NW), 0, s, (const float*)q, ldq,
                        (const float*)k_pages, (const float*)v_pages, page_size, table, table_stride,
-                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (float*)out, ldo);
+                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (float*)out, ldo, part);
+    if (n_runs > 1)
+      hipLaunchKernelGGL(talk_combine_kernel<float>, dim3(n_blocks / n_runs, H), dim3(64), 0, s, part, n_runs,
+                         (const SeqMeta*)seqs, (float*)out, ldo);
   } else if (dtype == kBF16) {
     LS_REQUIRE(ldq % 8 == 0, "talk_attention: query rows must be 16-byte aligned");
     hipLaunchKernelGGL(talk_attention_kernel<bf16_t>, dim3(n_blocks), dim3(64 * NW), 0, s, (const bf16_t*)q, ldq,
                        (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_size, table, table_stride,
-                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (bf16_t*)out, ldo);
+                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (bf16_t*)out, ldo, part);
+    if (n_runs > 1)
+      hipLaunchKernelGGL(talk_combine_kernel<bf16_t>, dim3(n_blocks / n_runs, H), dim3(64), 0, s, part, n_runs,
+                         (const SeqMeta*)seqs, (bf16_t*)out, ldo);
   } else {
     return fail("talk_attention: unknown dtype %d", dtype);
   }

@@ -233,7 +233,7 @@ def build_attention_mutants(head_dim: int, force: bool = False) -> Path:
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
 MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the controls
 #: (query heads, kv heads, key size, value size) of the talking-heads attention the tests and measurements use
-DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128), (32, 8, 128, 128))
+DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128))
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True,

@@ -809,17 +809,25 @@ class Kernels:
 
     def talk_attention(self, q: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, k_pages, v_pages,
                        page_size: int, table, seqs, blocks: torch.Tensor, n_blocks: int, talk: torch.Tensor,
-                       scale: float, window: int, keep_first: int, out: torch.Tensor) -> None:
+                       scale: float, window: int, keep_first: int, out: torch.Tensor, n_runs: int = 1,
+                       part: torch.Tensor | None = None) -> None:
         """Talking-heads attention of the step's queries ``q [T, heads*dim]`` over the paged cache; ``blocks``
-        lists ``n_blocks`` pairs (request of the step, block of 16 of its rows); ``talk [heads, heads]``."""
+        lists ``n_blocks`` work items of four ints (request of the step, block of 16 of its rows, run, runs);
+        ``talk [heads, heads]``.  ``n_runs > 1`` (single decoded tokens only): request i's visible keys are dealt
+        to its items ``i * n_runs ..`` in contiguous runs, whose results ``part`` (float32, ``n_blocks * heads *
+        (vdim + 2)`` elements) holds until a second launch has folded them."""
         lib = self.talking_lib(heads, kv_heads, dim, vdim)
         _rows_ok(q, "talk_attention q"); _rows_ok(out, "talk_attention out")
         if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype and q.shape[1] == heads * dim
                 and out.shape[1] == heads * vdim and out.shape[0] == q.shape[0]):
             raise KernelError("talk_attention q / out have the wrong shape or dtype")
         self._paged_ok(k_pages, v_pages, table, q.dtype, kv_heads, page_size, dim, vdim)
-        if not (blocks.is_cuda and blocks.dtype == torch.int32 and blocks.is_contiguous() and blocks.numel() >= 2 * n_blocks):
-            raise KernelError("talk_attention blocks must hold two int32 each")
+        if not (blocks.is_cuda and blocks.dtype == torch.int32 and blocks.is_contiguous() and blocks.numel() >= 4 * n_blocks):
+            raise KernelError("talk_attention work items must hold four int32 each")
+        if n_runs > 1 and not (part is not None and part.is_cuda and part.dtype == torch.float32 and part.is_contiguous()
+                               and part.numel() >= n_blocks * heads * (vdim + 2) and n_blocks % n_runs == 0
+                               and q.shape[0] * n_runs == n_blocks):
+            raise KernelError("talk_attention runs: one token a request, n_runs items a request and room for their results")
         self._f32_vector(talk, heads * heads, "talk_attention talk")
         if not (window > 0 and keep_first >= 0):
             raise KernelError(f"talk_attention window {window} / kept first tokens {keep_first}")
@@ -828,22 +836,29 @@ class Kernels:
         self._launch(lib, lib.ls_talk_attention, (
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
             _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(blocks), c_int(n_blocks), _ptr(talk), c_float(scale),
-            c_int(window), c_int(keep_first), _ptr(out), c_long(out.stride(0)), _stream()))
+            c_int(window), c_int(keep_first), _ptr(out), c_long(out.stride(0)), c_int(n_runs), _ptr(part), _stream()))
 
     LINREC_HGRN2, LINREC_RETENTION = 0, 1
 
     def linrec_max_dim(self) -> int:
         return self._memo(("linrec_max_dim",), lambda: int(self.mixers_lib().ls_linrec_max_dim()))
 
+    def linrec_gate_floats(self, n_tokens: int, heads: int, dim: int) -> int:
+        """Floats of the scratch buffer ``linrec`` needs for a step of ``n_tokens`` tokens."""
+        lib = self.mixers_lib()
+        lib.ls_linrec_gate_floats.restype = ctypes.c_long
+        return int(lib.ls_linrec_gate_floats(c_int(n_tokens), c_int(heads), c_int(dim)))
+
     def linrec(self, mode: int, raw: torch.Tensor, q_at: int, ab_at: int, v_at: int, heads: int, dim: int, vdim: int,
-               p0, p1, cos, sin, rot: int, max_pos: int, seqs, n_seqs: int, state: torch.Tensor,
-               out: torch.Tensor) -> None:
+               p0, p1, cos, sin, rot: int, max_pos: int, tok_pos, seqs, n_seqs: int, state: torch.Tensor,
+               gates: torch.Tensor, out: torch.Tensor) -> None:
         """The linear recurrence ``S_t = diag(a_t) S_(t-1) + b_t v_t^T``, ``o_t = S_t^T q_t`` over the tokens of
         every request of the step; ``raw`` float32 holds the projections (q at column ``q_at``, the gate or key
         projection at ``ab_at``, v at ``v_at``), ``state`` float32 ``[slots, heads, dim, vdim]`` is read and
         left for the next step, ``out`` float32 ``[T, heads*vdim]`` gets ``o_t``.  Mode ``LINREC_HGRN2``:
         ``p0`` lower bounds ``[heads*dim]``, ``p1`` the gate's bias or None; ``LINREC_RETENTION``: ``p0`` the
-        heads' decays, rotation tables for q and k."""
+        heads' decays, rotation tables for q and k at the positions ``tok_pos``.  ``gates``: float32 scratch of
+        ``linrec_gate_floats`` elements (q, decay and write gate of every token, computed once a step)."""
         _rows_ok(raw, "linrec raw"); _rows_ok(out, "linrec out")
         if not (raw.dtype == torch.float32 and out.dtype == torch.float32 and out.shape[1] == heads * vdim
                 and out.shape[0] == raw.shape[0]):
@@ -864,13 +879,19 @@ class Kernels:
         else:
             self._f32_vector(p0, heads, "linrec decays")
             positions = self._rotation_tables(cos, sin, rot, max_pos)
+        if not (gates.is_cuda and gates.dtype == torch.float32 and gates.is_contiguous()
+                and gates.numel() >= self.linrec_gate_floats(raw.shape[0], heads, dim)):
+            raise KernelError("linrec gates: float32 scratch of linrec_gate_floats elements")
+        if not (tok_pos.is_cuda and tok_pos.dtype == torch.int32 and tok_pos.is_contiguous() and tok_pos.numel() >= raw.shape[0]):
+            raise KernelError("linrec tok_pos: int32, one position a token")
         if n_seqs == 0 or raw.shape[0] == 0:
             return
         lib = self.mixers_lib()
         self._launch(lib, lib.ls_linrec, (
-            c_int(mode), _ptr(raw), c_long(raw.stride(0)), c_int(q_at), c_int(ab_at), c_int(v_at), c_int(heads),
-            c_int(dim), c_int(vdim), _ptr(p0), _ptr(p1), _ptr(cos), _ptr(sin), c_int(rot), c_int(positions),
-            c_int(max_pos), _ptr(seqs), c_int(n_seqs), _ptr(state), _ptr(out), c_long(out.stride(0)), _stream()))
+            c_int(mode), _ptr(raw), c_long(raw.stride(0)), c_int(q_at), c_int(ab_at), c_int(v_at), c_int(raw.shape[0]),
+            c_int(heads), c_int(dim), c_int(vdim), _ptr(p0), _ptr(p1), _ptr(cos), _ptr(sin), c_int(rot),
+            c_int(positions), c_int(max_pos), _ptr(tok_pos), _ptr(seqs), c_int(n_seqs), _ptr(state), _ptr(gates),
+            _ptr(out), c_long(out.stride(0)), _stream()))
 
     def head_norm_gate(self, x: torch.Tensor, heads: int, vdim: int, weight, gate, eps: float, out: torch.Tensor) -> None:
         """Per (token, head): ``x / sqrt(mean(x^2) + eps)`` over the head's ``vdim`` values, times ``weight

@@ -88,8 +88,9 @@ class HGRN2(_LinearRecurrence):
         raw = ctx.buf("recurrence.in_f32", (t, 2 * n * d + n * dv), torch.float32)
         k.gemm(x, self.w_in, raw, STORE_F32)
         o = ctx.buf("recurrence.o_f32", (t, n * dv), torch.float32)
+        gates = ctx.buf("recurrence.gates", (k.linrec_gate_floats(t, n, d),), torch.float32)
         k.linrec(k.LINREC_HGRN2, raw, 0, n * d, 2 * n * d, n, d, dv, self.lower, self.f_bias, None, None, 0,
-                 ctx.max_position, ctx.seqs, ctx.n_seqs, ctx.cache.unit_state(run.cache), o)
+                 ctx.max_position, ctx.tok_pos, ctx.seqs, ctx.n_seqs, ctx.cache.unit_state(run.cache), gates, o)
         normed = ctx.buf("recurrence.normed", (t, n * dv), rt.dtype)
         k.head_norm_gate(o, n, dv, self.norm, None, self.eps, normed)
         return project_out(ctx, normed, self.w_o, out, accumulate, defer, "recurrence.out_slices")
@@ -146,9 +147,10 @@ class Retention(_LinearRecurrence):
         raw = ctx.buf("recurrence.in_f32", (t, 2 * n * d + 2 * n * dv), torch.float32)
         k.gemm(x, self.w_in, raw, STORE_F32)
         o = ctx.buf("recurrence.o_f32", (t, n * dv), torch.float32)
+        gates = ctx.buf("recurrence.gates", (k.linrec_gate_floats(t, n, d),), torch.float32)
         k.linrec(k.LINREC_RETENTION, raw, 0, n * d, 2 * n * d, n, d, dv, self.decays, None, self.position.cos,
-                 self.position.sin, self.position.rotary_dim, ctx.max_position, ctx.seqs, ctx.n_seqs,
-                 ctx.cache.unit_state(run.cache), o)
+                 self.position.sin, self.position.rotary_dim, ctx.max_position, ctx.tok_pos, ctx.seqs, ctx.n_seqs,
+                 ctx.cache.unit_state(run.cache), gates, o)
         gated = ctx.buf("recurrence.normed", (t, n * dv), rt.dtype)
         k.head_norm_gate(o, n, dv, None, raw[:, 2 * n * d + n * dv:], self.eps, gated)
         return project_out(ctx, gated, self.w_o, out, accumulate, defer, "recurrence.out_slices")

@@ -29,6 +29,8 @@ from ..ops import STORE_F32
 from .base import Mixer, PagedKVSpec, WeightSpec, build_part, project_out, register_part
 
 ROWS_A_BLOCK = 16      # query rows of a work item of the attention kernel
+TILE_KEYS = 32         # keys of a tile of the attention kernel
+MAX_RUNS = 16          # the most runs the keys of a decoded token are dealt to
 
 
 @register_part("talking_attention")
@@ -114,16 +116,25 @@ class TalkingAttention(Mixer):
         key = ("talking_attention", "blocks")
         if ctx.declared(key):
             return
-        # work items: (request of the step, block of its rows); single decoded tokens are one block each
+        # work items: (request of the step, block of its rows, run, runs)
+        runs = 1
         if ctx.single_tokens:
-            pairs = np.stack([np.arange(ctx.n_seqs), np.zeros(ctx.n_seqs, dtype=np.int64)], axis=1)
+            # one row block a request: deal its visible keys to several items while the GPU has room for them
+            # (a number of runs that many steps share: it depends on the number of requests and on a power of
+            # two above the longest context only)
+            longest = int(ctx.kv_len.max()) + ctx.horizon
+            tiles = 1 << max(0, (-(-longest // TILE_KEYS) - 1).bit_length())
+            room = max(1, (2 * ctx.rt.kernels.compute_units()) // ctx.n_seqs)
+            runs = max(1, min(MAX_RUNS, room, tiles // 4))
+            seq = np.repeat(np.arange(ctx.n_seqs), runs)
+            items = np.stack([seq, np.zeros_like(seq), np.tile(np.arange(runs), ctx.n_seqs), np.full_like(seq, runs)], axis=1)
         else:
             counts = -(-ctx.q_len // ROWS_A_BLOCK)
             seq = np.repeat(np.arange(ctx.n_seqs), counts)
             first = np.repeat(np.cumsum(counts) - counts, counts)
-            pairs = np.stack([seq, np.arange(int(counts.sum())) - first], axis=1)
-        ctx.declare(key, pairs.reshape(-1), signature=("talking_attention", len(pairs)))
-        ctx.notes[key] = len(pairs)
+            items = np.stack([seq, np.arange(int(counts.sum())) - first, np.zeros_like(seq), np.ones_like(seq)], axis=1)
+        ctx.declare(key, items.reshape(-1), signature=("talking_attention", len(items), runs))
+        ctx.notes[key] = (len(items), runs)
 
     def forward(self, ctx, run, x, out, accumulate: bool, defer: bool = False):
         rt = ctx.rt
@@ -145,6 +156,8 @@ class TalkingAttention(Mixer):
                    group.page_size, {None: 0, "source": 1, "mix": 2}[self.v_mix], self.vmix, v_first)
         key = ("talking_attention", "blocks")
         attn = ctx.buf("talking.out", (t, nq * dv), rt.dtype)
+        n_items, runs = ctx.notes[key]
+        part = ctx.buf("talking.part", (n_items * nq * (dv + 2),), torch.float32) if runs > 1 else None
         k.talk_attention(q, nq, nkv, d, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
-                         ctx.block(key), ctx.notes[key], self.talk, self.scale, self.window, self.keep_first, attn)
+                         ctx.block(key), n_items, self.talk, self.scale, self.window, self.keep_first, attn, runs, part)
         return project_out(ctx, attn, self.w_o, out, accumulate, defer, "talking.out_slices")

@@ -124,6 +124,7 @@ class _Seqs:
             rows.append([at, n, s, s + n, slot, 0, 0, 0])
             at += n
         self.dev = torch.tensor(rows, dtype=torch.int32).reshape(-1).cuda()
+        self.positions = torch.tensor([s + i for n, s in zip(lengths, starts) for i in range(n)], dtype=torch.int32).cuda()
         self.n = len(lengths)
 
 
@@ -155,8 +156,9 @@ def test_recurrence_kernel_both_modes_over_unequal_requests_in_two_steps(heads, 
             raw = torch.cat([raws[i][starts[i]:starts[i] + lengths[i]] for i in live]).cuda()
             out = torch.empty(raw.shape[0], heads * vdim, device="cuda")
             p0, p1 = (lower.cuda(), f_bias.cuda()) if mode == K().LINREC_HGRN2 else (decay.cuda(), None)
+            gates = torch.empty(K().linrec_gate_floats(raw.shape[0], heads, dim), device="cuda")
             K().linrec(mode, raw, 0, heads * dim, 2 * heads * dim, heads, dim, vdim, p0, p1, cos, sin, rot, 63,
-                       seqs.dev, seqs.n, state, out)
+                       seqs.positions, seqs.dev, seqs.n, state, gates, out)
             at = 0
             for i in live:
                 got[i].append(out[at:at + lengths[i]].cpu())
