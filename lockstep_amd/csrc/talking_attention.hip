@@ -20,10 +20,11 @@
 //      (row statistics over the four lanes that share a query row);
 //   3. O^T += V^T P^T per head with the atom (value columns are the first operand, so the lane
 //      that holds a row's statistics also holds the row's accumulators).
-// A step of single decoded tokens has one row block a request, which would leave most of the GPU
-// idle while one workgroup walks the whole window: there a request's tiles are dealt to several work
-// items in contiguous runs, each leaves (max, sum, unnormalised output) of its run for the request's
-// one row, and a second kernel folds the runs in ascending order.
+// One workgroup that walks all visible keys of a row block would leave most of the GPU idle (a step
+// of decoded tokens has one row block a request; the late row blocks of a long prompt see many
+// times the keys of the early ones): a row block's tiles are dealt to several work items in
+// contiguous runs, each leaves (max, sum, unnormalised output) of its run for every row, and a
+// second kernel folds the runs in ascending order.
 // Scores, weights, statistics and accumulators are float; products read the compute dtype T.
 // Keys a request does not hold (beyond its length, pages a window has released) enter as zeros and
 // are masked; their values are replaced by zeros before the product.
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
     const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ blocks,
     const float* __restrict__ talk, float scale, int window, int keep_first, T* __restrict__ out, long ldo,
-    float* __restrict__ part) {
+    float* __restrict__ part, int part_rows) {
   constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
   constexpr int KCH = (D + KC - 1) / KC;  // chunks of a key (lanes beyond D in the last one bring zeros)
   __shared__ f32x4 raw_s[H][2][64];  // [head][half of the tile][lane]: the lane's four keys of that half
@@ -260,11 +261,11 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
   }
   if (!row_ok) return;
   if (n_runs > 1) {
-    // (single decoded tokens: row 0 only) [item][head][DV + 2]: the unnormalised output, then max and sum
-    if (l16 != 0) return;
+    // [item][row][head][DV + 2]: the unnormalised output, then max and sum (part_rows 1: decoded tokens, row 0 only)
+    if (l16 >= part_rows) return;
 #pragma unroll
     for (int x = 0; x < HPW; ++x) {
-      float* dst = part + ((long)blockIdx.x * H + w * HPW + x) * (DV + 2);
+      float* dst = part + (((long)blockIdx.x * part_rows + l16) * H + w * HPW + x) * (DV + 2);
 #pragma unroll
       for (int b = 0; b < VB; ++b)
 #pragma unroll
@@ -290,26 +291,29 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
   }
 }
 
-// Fold the runs of a decoded token: for request `seq` (one row) and head h, the partial results of the
-// items seq * n_runs .. seq * n_runs + n_runs - 1 in ascending order.  One workgroup a (request, head).
+// Fold the runs of row blocks: a fold item (first work item, runs, first packed row, rows) names the work items
+// first .. first + runs - 1 of one row block, whose partial results are folded in ascending order for each of its
+// rows.  One workgroup a (fold item, head).
 template <typename T>
-__global__ __launch_bounds__(64) void talk_combine_kernel(const float* __restrict__ part, int n_runs,
-                                                          const SeqMeta* __restrict__ seqs, T* __restrict__ out,
+__global__ __launch_bounds__(64) void talk_combine_kernel(const float* __restrict__ part, int part_rows,
+                                                          const int* __restrict__ folds, T* __restrict__ out,
                                                           long ldo) {
-  const int seq = blockIdx.x, h = blockIdx.y;
-  const SeqMeta m = seqs[seq];
-  if (m.q_len <= 0) return;
-  const float* mine = part + ((long)seq * n_runs * H + h) * (DV + 2);
-  const long stride = (long)H * (DV + 2);
-  float top = kNegSentinel;
-  for (int r = 0; r < n_runs; ++r) top = fmaxf(top, mine[r * stride + DV]);
-  float total = 0.f;
-  for (int r = 0; r < n_runs; ++r) total = total + mine[r * stride + DV + 1] * softmax_exp<T>(mine[r * stride + DV] - top);
-  const float inv = 1.0f / total;
-  for (int c = threadIdx.x; c < DV; c += 64) {
-    float sum = 0.f;
-    for (int r = 0; r < n_runs; ++r) sum = sum + mine[r * stride + c] * softmax_exp<T>(mine[r * stride + DV] - top);
-    out[(long)m.q_off * ldo + h * DV + c] = from_f32<T>(sum * inv);
+  const int first = folds[4 * blockIdx.x], n_runs = folds[4 * blockIdx.x + 1];
+  const int row0 = folds[4 * blockIdx.x + 2], rows = folds[4 * blockIdx.x + 3];
+  const int h = blockIdx.y;
+  const long stride = (long)part_rows * H * (DV + 2);  // from a run to the next
+  for (int r = 0; r < rows; ++r) {
+    const float* mine = part + (((long)first * part_rows + r) * H + h) * (DV + 2);
+    float top = kNegSentinel;
+    for (int k = 0; k < n_runs; ++k) top = fmaxf(top, mine[k * stride + DV]);
+    float total = 0.f;
+    for (int k = 0; k < n_runs; ++k) total = total + mine[k * stride + DV + 1] * softmax_exp<T>(mine[k * stride + DV] - top);
+    const float inv = 1.0f / total;
+    for (int c = threadIdx.x; c < DV; c += 64) {
+      float sum = 0.f;
+      for (int k = 0; k < n_runs; ++k) sum = sum + mine[k * stride + c] * softmax_exp<T>(mine[k * stride + DV] - top);
+      out[(long)(row0 + r) * ldo + h * DV + c] = from_f32<T>(sum * inv);
+    }
   }
 }
 
@@ -327,14 +331,16 @@ extern "C" int ls_talk_vdim() { return DV; }
 // q [T][ldq] (rotated queries, H heads of D); key pages [pages][G][page_size][D], value pages
 // [pages][G][DV][page_size]; table [slots][table_stride]; seqs: the step's requests; blocks: n_blocks work items
 // of four ints (request of the step, block of 16 of its rows, run, runs); talk [H][H] float; out [T][ldo] (H heads
-// of DV).  n_runs > 1: a step of single decoded tokens whose request i has the items i * n_runs .. (one a run);
-// part then holds n_blocks * H * (DV + 2) floats, and a second launch folds the runs into out.
+// of DV).  Work items with runs > 1 leave their results in part (n_blocks * part_rows * H * (DV + 2) floats;
+// part_rows 16, or 1 for a step of single decoded tokens) and the n_folds fold items of four ints (first work
+// item, runs, first packed row, rows) say which to fold into which rows of out in a second launch.
 extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages,
                                  int page_size, const int* table, int table_stride, const void* seqs,
                                  const int* blocks, int n_blocks, const float* talk, float scale, int window,
-                                 int keep_first, void* out, long ldo, int n_runs, float* part, void* stream) {
-  LS_REQUIRE(n_runs >= 1 && (n_runs == 1 || (part && n_blocks % n_runs == 0)), "talk_attention: %d runs over %d items",
-             n_runs, n_blocks);
+                                 int keep_first, void* out, long ldo, const int* folds, int n_folds, float* part,
+                                 int part_rows, void* stream) {
+  LS_REQUIRE(n_folds >= 0 && (n_folds == 0 || (part && folds && (part_rows == 1 || part_rows == 16))),
+             "talk_attention: %d fold items need partial results of 1 or 16 rows", n_folds);
   LS_REQUIRE(n_blocks > 0 && q && k_pages && v_pages && table && seqs && blocks && talk && out, "talk_attention: null operand");
   LS_REQUIRE(ldq >= (long)H * D && ldo >= (long)H * DV, "talk_attention: rows are too short");
   LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && table_stride > 0, "talk_attention: page size %d", page_size);
@@ -347,18 +353,19 @@ extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void*
     LS_REQUIRE(ldq % 4 == 0, "talk_attention: query rows must be 16-byte aligned");
     hipLaunchKernelGGL(talk_attention_kernel<float>, dim3(n_blocks), dim3(64 * NW), 0, s, (const float*)q, ldq,
                        (const float*)k_pages, (const float*)v_pages, page_size, table, table_stride,
-                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (float*)out, ldo, part);
-    if (n_runs > 1)
-      hipLaunchKernelGGL(talk_combine_kernel<float>, dim3(n_blocks / n_runs, H), dim3(64), 0, s, part, n_runs,
-                         (const SeqMeta*)seqs, (float*)out, ldo);
+                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (float*)out, ldo, part, part_rows);
+    if (n_folds > 0)
+      hipLaunchKernelGGL(talk_combine_kernel<float>, dim3(n_folds, H), dim3(64), 0, s, part, part_rows, folds,
+                         (float*)out, ldo);
   } else if (dtype == kBF16) {
     LS_REQUIRE(ldq % 8 == 0, "talk_attention: query rows must be 16-byte aligned");
     hipLaunchKernelGGL(talk_attention_kernel<bf16_t>, dim3(n_blocks), dim3(64 * NW), 0, s, (const bf16_t*)q, ldq,
                        (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_size, table, table_stride,
-                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (bf16_t*)out, ldo, part);
-    if (n_runs > 1)
-      hipLaunchKernelGGL(talk_combine_kernel<bf16_t>, dim3(n_blocks / n_runs, H), dim3(64), 0, s, part, n_runs,
-                         (const SeqMeta*)seqs, (bf16_t*)out, ldo);
+                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (bf16_t*)out, ldo, part,
+                       part_rows);
+    if (n_folds > 0)
+      hipLaunchKernelGGL(talk_combine_kernel<bf16_t>, dim3(n_folds, H), dim3(64), 0, s, part, part_rows, folds,
+                         (bf16_t*)out, ldo);
   } else {
     return fail("talk_attention: unknown dtype %d", dtype);
   }

@@ -809,13 +809,14 @@ class Kernels:
 
     def talk_attention(self, q: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, k_pages, v_pages,
                        page_size: int, table, seqs, blocks: torch.Tensor, n_blocks: int, talk: torch.Tensor,
-                       scale: float, window: int, keep_first: int, out: torch.Tensor, n_runs: int = 1,
-                       part: torch.Tensor | None = None) -> None:
+                       scale: float, window: int, keep_first: int, out: torch.Tensor, folds: torch.Tensor | None = None,
+                       n_folds: int = 0, part: torch.Tensor | None = None, part_rows: int = 16) -> None:
         """Talking-heads attention of the step's queries ``q [T, heads*dim]`` over the paged cache; ``blocks``
         lists ``n_blocks`` work items of four ints (request of the step, block of 16 of its rows, run, runs);
-        ``talk [heads, heads]``.  ``n_runs > 1`` (single decoded tokens only): request i's visible keys are dealt
-        to its items ``i * n_runs ..`` in contiguous runs, whose results ``part`` (float32, ``n_blocks * heads *
-        (vdim + 2)`` elements) holds until a second launch has folded them."""
+        ``talk [heads, heads]``.  A row block whose visible keys are dealt to several work items (runs > 1) has a
+        fold item of four ints in ``folds`` (first work item, runs, first packed row, rows); their results wait in
+        ``part`` (float32, ``n_blocks * part_rows * heads * (vdim + 2)`` elements; ``part_rows`` 16, or 1 for a step
+        of single decoded tokens) until a second launch has folded them."""
         lib = self.talking_lib(heads, kv_heads, dim, vdim)
         _rows_ok(q, "talk_attention q"); _rows_ok(out, "talk_attention out")
         if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype and q.shape[1] == heads * dim
@@ -824,10 +825,12 @@ class Kernels:
         self._paged_ok(k_pages, v_pages, table, q.dtype, kv_heads, page_size, dim, vdim)
         if not (blocks.is_cuda and blocks.dtype == torch.int32 and blocks.is_contiguous() and blocks.numel() >= 4 * n_blocks):
             raise KernelError("talk_attention work items must hold four int32 each")
-        if n_runs > 1 and not (part is not None and part.is_cuda and part.dtype == torch.float32 and part.is_contiguous()
-                               and part.numel() >= n_blocks * heads * (vdim + 2) and n_blocks % n_runs == 0
-                               and q.shape[0] * n_runs == n_blocks):
-            raise KernelError("talk_attention runs: one token a request, n_runs items a request and room for their results")
+        if n_folds:
+            if not (folds is not None and folds.is_cuda and folds.dtype == torch.int32 and folds.is_contiguous()
+                    and folds.numel() >= 4 * n_folds and part_rows in (1, 16)
+                    and part is not None and part.is_cuda and part.dtype == torch.float32 and part.is_contiguous()
+                    and part.numel() >= n_blocks * part_rows * heads * (vdim + 2)):
+                raise KernelError("talk_attention folds: four int32 each, and room for every work item's partial result")
         self._f32_vector(talk, heads * heads, "talk_attention talk")
         if not (window > 0 and keep_first >= 0):
             raise KernelError(f"talk_attention window {window} / kept first tokens {keep_first}")
@@ -836,7 +839,8 @@ class Kernels:
         self._launch(lib, lib.ls_talk_attention, (
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
             _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(blocks), c_int(n_blocks), _ptr(talk), c_float(scale),
-            c_int(window), c_int(keep_first), _ptr(out), c_long(out.stride(0)), c_int(n_runs), _ptr(part), _stream()))
+            c_int(window), c_int(keep_first), _ptr(out), c_long(out.stride(0)), _ptr(folds), c_int(n_folds), _ptr(part),
+            c_int(part_rows), _stream()))
 
     LINREC_HGRN2, LINREC_RETENTION = 0, 1
 

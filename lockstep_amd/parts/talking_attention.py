@@ -30,7 +30,8 @@ from .base import Mixer, PagedKVSpec, WeightSpec, build_part, project_out, regis
 
 ROWS_A_BLOCK = 16      # query rows of a work item of the attention kernel
 TILE_KEYS = 32         # keys of a tile of the attention kernel
-MAX_RUNS = 16          # the most runs the keys of a decoded token are dealt to
+MAX_RUNS = 16          # the most runs the keys of a row block are dealt to
+TILES_A_RUN = 8        # a row block of a prompt portion is cut into runs of at least this many tiles
 
 
 @register_part("talking_attention")
@@ -109,32 +110,58 @@ class TalkingAttention(Mixer):
 
     def prepare_group(self):
         share = getattr(self.position, "share_key", None)
-        return None if share is None else ("talking_attention", share())
+        return None if share is None else ("talking_attention", self.window, self.keep_first, share())
+
+    def _block_key(self):
+        return ("talking_attention", "work", self.window, self.keep_first)
 
     def prepare(self, ctx) -> None:
+        """The step's work items, shared by the layers with this window and these kept tokens: (request of the
+        step, block of its rows, run, runs), and the fold items of the row blocks that were cut into runs."""
         self.position.ensure(ctx.max_position + 1, ctx.rt)
-        key = ("talking_attention", "blocks")
+        key = self._block_key()
         if ctx.declared(key):
             return
-        # work items: (request of the step, block of its rows, run, runs)
-        runs = 1
+        cus = ctx.rt.kernels.compute_units()
         if ctx.single_tokens:
             # one row block a request: deal its visible keys to several items while the GPU has room for them
             # (a number of runs that many steps share: it depends on the number of requests and on a power of
             # two above the longest context only)
-            longest = int(ctx.kv_len.max()) + ctx.horizon
+            longest = min(int(ctx.kv_len.max()) + ctx.horizon, self.window + self.keep_first)
             tiles = 1 << max(0, (-(-longest // TILE_KEYS) - 1).bit_length())
-            room = max(1, (2 * ctx.rt.kernels.compute_units()) // ctx.n_seqs)
-            runs = max(1, min(MAX_RUNS, room, tiles // 4))
+            runs = max(1, min(MAX_RUNS, (2 * cus) // ctx.n_seqs, tiles // 4))
             seq = np.repeat(np.arange(ctx.n_seqs), runs)
             items = np.stack([seq, np.zeros_like(seq), np.tile(np.arange(runs), ctx.n_seqs), np.full_like(seq, runs)], axis=1)
+            rows = np.arange(ctx.n_seqs)            # a request's one row is packed row i
+            folds = np.stack([rows * runs, np.full_like(rows, runs), rows, np.ones_like(rows)], axis=1) if runs > 1 else None
+            part_rows = 1
         else:
             counts = -(-ctx.q_len // ROWS_A_BLOCK)
             seq = np.repeat(np.arange(ctx.n_seqs), counts)
-            first = np.repeat(np.cumsum(counts) - counts, counts)
-            items = np.stack([seq, np.arange(int(counts.sum())) - first, np.zeros_like(seq), np.ones_like(seq)], axis=1)
-        ctx.declare(key, items.reshape(-1), signature=("talking_attention", len(items), runs))
-        ctx.notes[key] = (len(items), runs)
+            block = np.arange(int(counts.sum())) - np.repeat(np.cumsum(counts) - counts, counts)
+            first = ctx.q_start[seq] + block * ROWS_A_BLOCK                       # position of a block's first row
+            rows = np.minimum(ROWS_A_BLOCK, ctx.q_len[seq] - block * ROWS_A_BLOCK)
+            last = first + rows - 1
+            # the tiles a block walks: the kept ones below the window's first, then the window's (as the kernel counts)
+            lo = np.maximum(0, first - self.window + 1) // TILE_KEYS
+            kept = np.minimum(-(-self.keep_first // TILE_KEYS), lo)
+            tiles = kept + last // TILE_KEYS - lo + 1
+            # runs of at least TILES_A_RUN tiles, longer where the step has more work than a few items a CU
+            a_run = max(TILES_A_RUN, -(-int(tiles.sum()) // (4 * cus)))
+            runs = np.minimum(MAX_RUNS, np.maximum(1, tiles // a_run))
+            item_block = np.repeat(np.arange(len(seq)), runs)
+            run = np.arange(int(runs.sum())) - np.repeat(np.cumsum(runs) - runs, runs)
+            items = np.stack([seq[item_block], block[item_block], run, runs[item_block]], axis=1)
+            cut = runs > 1
+            folds = None
+            if cut.any():
+                first_item = (np.cumsum(runs) - runs)[cut]
+                folds = np.stack([first_item, runs[cut], (ctx.q_off[seq] + block * ROWS_A_BLOCK)[cut], rows[cut]], axis=1)
+            part_rows = ROWS_A_BLOCK
+        n_folds = 0 if folds is None else len(folds)
+        ints = items.reshape(-1) if folds is None else np.concatenate([items.reshape(-1), folds.reshape(-1)])
+        ctx.declare(key, ints, signature=("talking_attention", len(items), n_folds, part_rows))
+        ctx.notes[key] = (len(items), n_folds, part_rows)
 
     def forward(self, ctx, run, x, out, accumulate: bool, defer: bool = False):
         rt = ctx.rt
@@ -154,10 +181,12 @@ class TalkingAttention(Mixer):
         k.talk_qkv(raw, t, nq, nkv, d, dv, self.b_qkv, self.position.cos, self.position.sin, self.position.rotary_dim,
                    ctx.max_position, ctx.tok_seq, ctx.tok_pos, ctx.seqs, group.table, q, key_pages, value_pages,
                    group.page_size, {None: 0, "source": 1, "mix": 2}[self.v_mix], self.vmix, v_first)
-        key = ("talking_attention", "blocks")
+        key = self._block_key()
         attn = ctx.buf("talking.out", (t, nq * dv), rt.dtype)
-        n_items, runs = ctx.notes[key]
-        part = ctx.buf("talking.part", (n_items * nq * (dv + 2),), torch.float32) if runs > 1 else None
+        n_items, n_folds, part_rows = ctx.notes[key]
+        work = ctx.block(key)
+        part = ctx.buf("talking.part", (n_items * part_rows * nq * (dv + 2),), torch.float32) if n_folds else None
         k.talk_attention(q, nq, nkv, d, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
-                         ctx.block(key), n_items, self.talk, self.scale, self.window, self.keep_first, attn, runs, part)
+                         work[:4 * n_items], n_items, self.talk, self.scale, self.window, self.keep_first, attn,
+                         work[4 * n_items:] if n_folds else None, n_folds, part, part_rows)
         return project_out(ctx, attn, self.w_o, out, accumulate, defer, "talking.out_slices")

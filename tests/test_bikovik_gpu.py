@@ -223,6 +223,22 @@ def test_whole_prompt_portions_and_token_by_token_agree_with_the_plain_model(mod
             assert rel_err(runs[label], runs["whole"]) < 1e-5, label
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_whose_late_row_blocks_are_cut_into_runs(models, dtype):
+    """A window of a thousand keys and a prompt of 700 tokens: the late row blocks of the prompt see
+    enough key tiles for the attention to deal them to several work items and fold the results (the
+    buffer of partial results exists afterwards); decoding goes on from there."""
+    model, oracle, raw, page, _ = models("B", dtype)
+    tokens = random_tokens(720, raw["vocab"], seed=13)
+    want = oracle.forward(tokens)
+    for cuts in ([700] + [1] * 20, [333, 2, 365] + [1] * 20):
+        cache = new_cache(model, page, tokens=1024)
+        got = feed(model, cache, "r", tokens, cuts)
+        assert rel_err(got, want) < TOL[dtype], cuts[:3]
+        cache.close("r")
+    assert any(name == "talking.part" for name, _, _ in model.workspace._buffers)
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_first_tokens_and_prompts_of_one_and_two_tokens(models, name):
     model, oracle, raw, page, _ = models(name)
