@@ -170,16 +170,16 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 // such), the four quarters of a column are neighbouring lanes and are added by exchanges inside the quad,
 // and the waves' parts are added in wave order.  The order of all sums is a function of D alone.
 //
-// The walk is software-pipelined over rounds of sixteen tokens, with two sets of LDS buffers: while
-// the waves walk the tokens of one round, the gates and values of the next are already requested
+// The walk is software-pipelined over chunks of sixteen tokens, with two sets of LDS buffers: while
+// the waves walk the tokens of one chunk, the gates and values of the next are already requested
 // (into registers); after the walk they are written to the other set, one barrier follows, and the
-// waves' parts of the round's o_t are added and stored while the next round is walked.
+// waves' parts of the chunk's o_t are added and stored while the next chunk is walked.
 // ---------------------------------------------------------------------------
 constexpr int kRecRows = 8;     // rows of the state a lane keeps
 constexpr int kRecCols = 16;    // columns of the state a workgroup takes
 constexpr int kRecWaveRows = 4 * kRecRows;  // rows a wave holds
 constexpr int kRecTokens = 16;  // tokens copied at a time
-constexpr int kRecPer = kRecTokens * 3 * kRecWaveRows / (4 * 64);  // vectors of four gates a thread copies a round
+constexpr int kRecPer = kRecTokens * 3 * kRecWaveRows / (4 * 64);  // vectors of four gates a thread copies a chunk
 constexpr int kRecVPer = kRecTokens * kRecCols / 64;                // the most values a thread fetches (one wave)
 
 __global__ __launch_bounds__(256) void linrec_gates_kernel(
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
 #pragma unroll
   for (int r = 0; r < kRecRows; ++r) S[r] = (row0 + r < D && col_ok) ? mine[(long)(row0 + r) * DV + c] : 0.f;
   const int v_per = (kRecTokens * kRecCols + (int)blockDim.x - 1) / (int)blockDim.x;
-  // a round's gates are kRecTokens * token consecutive floats of one head: token t at (t * H + head) * token.
+  // a chunk's gates are kRecTokens * token consecutive floats of one head: token t at (t * H + head) * token.
   // Thread i copies the vectors i, i + threads, ...; vector k lies in token k / (token / 4).
   const int vec_a_token = token / 4;
   int v_tt[kRecPer], v_in[kRecPer];
@@ -258,7 +258,7 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
     v_tt[j] = k / vec_a_token;
     v_in[j] = 4 * (k % vec_a_token);
   }
-  // the operands of the next round are requested before a round is walked
+  // the operands of the next chunk are requested before a chunk is walked
   f32x4 rg[kRecPer];
   float rv[kRecVPer];
 
@@ -290,8 +290,8 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
     }
   };
 
-  // one round: walk the tokens of the set `base`, leave the waves' parts of o_t there
-  auto walk_round = [&](float* base, int n) LS_INLINED {
+  // one chunk: walk the tokens of the set `base`, leave the waves' parts of o_t there
+  auto walk_chunk = [&](float* base, int n) LS_INLINED {
     const float* v_s = base + kRecTokens * token;
     float* o_s = base + kRecTokens * token + kRecTokens * kRecCols;  // [waves][tokens][columns]
     // a token's operands: eight q, a and b of the lane's rows (two vectors each) and its column's value
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
       if (quarter == 0) o_s[(g * kRecTokens + tt) * kRecCols + l16] = o;
     };
     if (n == kRecTokens) {
-      // a full round is unrolled, and the operands of the token after next are requested before a token is walked
+      // a full chunk is unrolled, and the operands of the token after next are requested before a token is walked
       Operands ahead = fetch(0), next = fetch(1);
 #pragma unroll
       for (int tt = 0; tt < kRecTokens; ++tt) {
@@ -336,9 +336,9 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
     }
   };
 
-  // the waves' parts of a round are added in wave order and stored (while the next round is walked: that round
-  // writes the other set, and the barrier at its end stands before the round after it writes this one again)
-  auto store_round = [&](const float* base, int t0, int n) LS_INLINED {
+  // the waves' parts of a chunk are added in wave order and stored (while the next chunk is walked: that chunk
+  // writes the other set, and the barrier at its end stands before the chunk after it writes this one again)
+  auto store_chunk = [&](const float* base, int t0, int n) LS_INLINED {
     const float* o_s = base + kRecTokens * token + kRecTokens * kRecCols;
     for (int idx = threadIdx.x; idx < n * kRecCols; idx += blockDim.x) {
       const int tt = idx / kRecCols, l = idx % kRecCols, col = cb * kRecCols + l;
@@ -356,10 +356,10 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
     const int n = min(kRecTokens, m.q_len - t0);
     const bool more = t0 + kRecTokens < m.q_len;
     if (more) request(t0 + kRecTokens);
-    walk_round(lds + at * set, n);
+    walk_chunk(lds + at * set, n);
     if (more) deposit(lds + (at ^ 1) * set);
     __syncthreads();
-    store_round(lds + at * set, t0, n);
+    store_chunk(lds + at * set, t0, n);
   }
 #pragma unroll
   for (int r = 0; r < kRecRows; ++r)
