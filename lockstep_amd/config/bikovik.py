@@ -91,7 +91,7 @@ class BikovikConfig(ModelConfig):
 
     # -- the mixers as parts ------------------------------------------------------------
     def _rotation(self, m, where: str) -> PartSpec:
-        if m.get("rot") is None:
+        if m.get("rot") is None or not m["rot"].get("dims"):
             return PartSpec("no_position", {})
         rot = m["rot"]
         dims = _positive_int(_need(rot, "dims", where + ".rot"), where + ".rot.dims")
