@@ -27,7 +27,18 @@ pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
 F64 = torch.float64
 
-TOL = {"float32": 3e-5, "bfloat16": 6e-2}      # of the largest logit of the request
+# Bounds on max |engine - plain| / max |plain logit| over a request, some three times the largest error
+# measured on the MI355X on these weights: float32 3.9e-6 (case B; the others below 1.1e-6); bfloat16 7.5e-3
+# (A), 2.0e-3 (C, one-layer attention), 1.1e-2 (one-layer HGRN2), 2.2e-3 (one-layer retention) and 3.3e-2 for
+# case B, whose soft cap of 8 makes the largest logit small and whose gated unit clamps at 0.7, where a
+# rounded bfloat16 input lands on the other side of the bound.  The cuttings of a request agree with each
+# other to all printed digits in both precisions.
+TOL = {"float32": 1.5e-5, "bfloat16": 3.5e-2}
+TOL_CASE = {("B", "bfloat16"): 1e-1}
+
+
+def tol(dtype, name=None):
+    return TOL_CASE.get((name, dtype), TOL[dtype])
 
 
 def K():
@@ -215,7 +226,7 @@ def test_whole_prompt_portions_and_token_by_token_agree_with_the_plain_model(mod
                         ("single", [1] * 150)):
         cache = new_cache(model, page)
         runs[label] = feed(model, cache, "r", tokens, cuts)
-        assert rel_err(runs[label], want) < TOL[dtype], (name, label)
+        assert rel_err(runs[label], want) < tol(dtype, name), (name, label)
         cache.close("r")
         cache.audit()
     if dtype == "float32":              # the cuttings agree with each other far below the bound against the plain model
@@ -234,7 +245,7 @@ def test_a_long_prompt_whose_late_row_blocks_are_cut_into_runs(models, dtype):
     for cuts in ([700] + [1] * 20, [333, 2, 365] + [1] * 20):
         cache = new_cache(model, page, tokens=1024)
         got = feed(model, cache, "r", tokens, cuts)
-        assert rel_err(got, want) < TOL[dtype], cuts[:3]
+        assert rel_err(got, want) < tol(dtype, "B"), cuts[:3]
         cache.close("r")
     assert any(name == "talking.part" for name, _, _ in model.workspace._buffers)
 
@@ -264,7 +275,7 @@ def test_mixed_batches_of_unequal_requests_with_pages_and_slots_used_again(model
     got = replay_in_process(model, cache, steps)
     assert cache.free_slots == 4 and all(g.pool.taken_total > g.pool.num_pages for g in cache.groups)
     for rid, toks in requests.items():
-        assert rel_err(got[rid], oracle.forward(toks)) < TOL[dtype], rid
+        assert rel_err(got[rid], oracle.forward(toks)) < tol(dtype, name), rid
 
 
 # ---------------------------------------------------------------------------
