@@ -442,3 +442,41 @@ def test_trace_replay_program_on_a_model_folder(models, tmp_path):
             at += len(e["want"])
     for rid, toks in requests.items():
         assert rel_err(np.concatenate(rows[rid]), oracle.forward(toks)) < TOL["float32"], rid
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_preempted_requests_recompute_state_and_pages_to_the_same_tokens(models, dtype):
+    """The scheduler preempts one request twice while two others run beside it (one of them draws
+    its tokens): its pages and its state slot are given back, its context runs again in portions
+    from an empty state, and every request's tokens and logits are those of the request alone."""
+    from lockstep_amd import Request, Scheduler
+    from lockstep_amd.engine.policy import PreemptAtStepsPolicy
+
+    model, oracle, raw, page, _ = models("A", dtype, seed=12)
+    vocab = raw["vocab"]
+    wave = [Request(uid="p0", prompt=random_tokens(2 * page + 3, vocab, seed=41), max_new_tokens=14),
+            Request(uid="p1", prompt=random_tokens(37, vocab, seed=42), max_new_tokens=9),
+            Request(uid="p2", prompt=random_tokens(5, vocab, seed=43), max_new_tokens=12, temperature=0.9, seed=7)]
+
+    def alone(request):
+        s = Scheduler(model, num_blocks=16, block_size=page, keep_logits=True, audit=False)
+        s.submit(Request(**vars(request)))
+        return s.run()[request.uid], torch.stack(s.emitted_logits[request.uid])
+
+    policy = PreemptAtStepsPolicy("p0", (5, 9), chunk=page + 3)
+    cache = model.make_cache(num_pages=40, page_size=page, max_requests=4, poison_on_free=True)
+    s = Scheduler(model, num_blocks=40, block_size=page, cache=cache, keep_logits=True, audit=True, policy=policy,
+                  max_batched_tokens=40)
+    for r in wave:
+        s.submit(Request(**vars(r)))
+    out = s.run()
+    s.counters.require_fired("preempt_fired", "resume", "prefill_chunk", "decode_step")
+    assert {q.uid: q.preemptions for q in s.done}["p0"] == 2
+    for r in wave:
+        tokens, rows = alone(r)
+        assert out[r.uid] == tokens, r.uid
+        assert rel_err(torch.stack(s.emitted_logits[r.uid]).cpu(), rows.cpu()) < 1e-5 if dtype == "float32" else True
+    if dtype == "float32":
+        assert out["p0"] == oracle.generate_greedy(wave[0].prompt, 14)
+    cache.audit()
+    assert cache.free_slots == 4
