@@ -345,10 +345,10 @@ def bikovik_like(qwen, layers: int, window: int = 4096, keep_first: int = 4):
     hgrn2 = {"type": "hgrn2", "mlp": mlp, "mixer": {"heads": heads, "dim": d, "vdim": d}}
     retention = {"type": "retention", "mlp": mlp, "mixer": {
         "heads": heads, "dim": d, "vdim": d, "rot": {"dims": d, "base": qwen.rope_theta},
-        "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, heads - 1)) for h in range(heads)]}}
+        "decay": [1.0 - 2.0 ** (-4.0 - 4.0 * h / max(1, heads - 1)) for h in range(heads)]}}
     cycle = [hgrn2, attention, retention, attention]
     return config_from_dict({"architecture": "Bikovik", "vocab": qwen.vocab_size, "width": qwen.hidden_size,
-                             "embedding": {"scale": 1.0}, "norm": {"eps": qwen.rms_norm_eps}, "logit_softcap": 30.0,
+                             "embedding": {"scale": 1.0}, "norm": {"eps": qwen.rms_norm_eps}, "logit_softcap": 50.0,
                              "layers": [cycle[i % 4] for i in range(layers)]})
 
 

@@ -205,7 +205,7 @@ def test_small_functions():
     want = [1.0 / (1 + torch.exp(torch.tensor(-1.702, dtype=F64))) * 2.0, -5.0 / (1 + torch.exp(torch.tensor(8.51, dtype=F64))) * 0.0,
             0.5 / (1 + torch.exp(torch.tensor(-0.851, dtype=F64))) * 1.25]
     assert torch.allclose(y, torch.stack([torch.as_tensor(w, dtype=F64) for w in want]))
-    assert torch.allclose(plain.soft_cap(torch.tensor([1e6, 0.1], dtype=F64), 30.0), torch.tensor([30.0, 30 * torch.tanh(torch.tensor(0.1 / 30, dtype=F64))], dtype=F64))
+    assert torch.allclose(plain.soft_cap(torch.tensor([1e6, 0.1], dtype=F64), 17.0), torch.tensor([17.0, 17 * torch.tanh(torch.tensor(0.1 / 17, dtype=F64))], dtype=F64))
     r = plain.root_mean_square_norm(torch.tensor([[3.0, 4.0]], dtype=F64), 0.0)
     assert torch.allclose(r, torch.tensor([[3.0, 4.0]], dtype=F64) / (12.5 ** 0.5))
 

@@ -75,7 +75,7 @@ def test_init_then_run_a_bikovik_folder(tmp_path):
                    check=True, capture_output=True, timeout=300)
     tensors = {name: handle.get(key) for name, (handle, key) in open_model_tensors(folder).items()}
     plain = PlainBikovik(json.loads((folder / "config.json").read_text()), tensors)
-    prompts = [random_tokens(n, 512, seed=90 + n) for n in (3, 21, 70)]
+    prompts = [random_tokens(n, 640, seed=90 + n) for n in (3, 21, 70)]
     want = {f"r{i:02d}": plain.generate_greedy(p, 6) for i, p in enumerate(prompts)}
     args = [x for p in prompts for x in ("--prompt-ids", ",".join(map(str, p)))]
     assert run("run", "--model", str(folder), "--dtype", "float32", "--max-new-tokens", "6", *args) == want
