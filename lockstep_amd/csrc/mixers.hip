@@ -219,6 +219,10 @@ __global__ __launch_bounds__(256) void linrec_gates_kernel(
   dst[2 * dp] = b;
 }
 
+// A barrier between the waves' LDS writes and reads that waits for this wave's LDS operations only: the global
+// loads of the next chunk stay on their way across it.
+__device__ __forceinline__ void lds_barrier() { __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Sum over the four neighbouring lanes 4k .. 4k + 3 (a DPP exchange inside the quad, no LDS traffic): first the
 // pairs (l, l ^ 1), then the pairs of pairs, so all four lanes end with the same bits.
 __device__ __forceinline__ float quad_sum(float v) {
@@ -350,7 +354,7 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
 
   request(0);
   deposit(lds);
-  __syncthreads();
+  lds_barrier();
   int at = 0;
   for (int t0 = 0; t0 < m.q_len; t0 += kRecTokens, at ^= 1) {
     const int n = min(kRecTokens, m.q_len - t0);
@@ -358,7 +362,7 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
     if (more) request(t0 + kRecTokens);
     walk_chunk(lds + at * set, n);
     if (more) deposit(lds + (at ^ 1) * set);
-    __syncthreads();
+    lds_barrier();
     store_chunk(lds + at * set, t0, n);
   }
 #pragma unroll

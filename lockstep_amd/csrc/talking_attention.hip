@@ -54,6 +54,11 @@ struct SeqMeta {
   int q_off, q_len, q_start, kv_len, table_row, reserved[3];
 };
 
+// A barrier between the waves' LDS writes and reads.  It waits for this wave's LDS operations only, not for its
+// global loads: the keys of the next tile stay on their way across it (the compiler still waits for a loaded
+// register before its first use).
+__device__ __forceinline__ void lds_barrier() { __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <typename T>
 __device__ __forceinline__ typename Atom<T>::vec_t load_or_zero(const T* p, bool ok) {
   typedef typename Atom<T>::vec_t vec_t;
@@ -106,51 +111,94 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
 
   const int per_run = (n_tiles + n_runs - 1) / n_runs;
   const int step_end = min(n_tiles, (run + 1) * per_run);
-  for (int step = run * per_run; step < step_end; ++step) {
-    const int tile = step < kept_tiles ? step : lo_tile + (step - kept_tiles);
-    const int key0 = tile * kTileKeys;
-    // -- 1. transposed raw scores of the wave's own heads ------------------------------------
-    // page and slot of the lane's key of each half (as a row of K), and of its four keys (as columns of V^T)
+
+  // A tile's keys are requested while the tile before it is worked on: its addresses (page and slot of the
+  // lane's key of each half as a row of K, and of its four keys as columns of V^T) and the key vectors of the
+  // key/value heads the wave reads.
+  struct Ahead {
     long k_at[2], v_at[2];
     bool k_ok[2], v_ok[2][4];
+    typename Atom<T>::vec_t kv[2][HPW / SH][KCH];
+  };
+  auto request = [&](int step, Ahead& t) LS_INLINED {
+    const int tile = step < kept_tiles ? step : lo_tile + (step - kept_tiles);
+    const int key0 = tile * kTileKeys;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int key = key0 + 16 * half + l16;
       const int page = key <= p_last ? my_table[key / page_size] : -1;
-      k_ok[half] = page >= 0;
-      k_at[half] = ((long)(page >= 0 ? page : 0) * G) * page_size + (page >= 0 ? key % page_size : 0);
+      t.k_ok[half] = page >= 0;
+      t.k_at[half] = ((long)(page >= 0 ? page : 0) * G) * page_size + (page >= 0 ? key % page_size : 0);
       const int key4 = key0 + 16 * half + 4 * quad;
       const int page4 = key4 <= p_last ? my_table[key4 / page_size] : -1;
-      v_at[half] = ((long)(page4 >= 0 ? page4 : 0) * G * DV) * page_size + (page4 >= 0 ? key4 % page_size : 0);
+      t.v_at[half] = ((long)(page4 >= 0 ? page4 : 0) * G * DV) * page_size + (page4 >= 0 ? key4 % page_size : 0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v_ok[half][i] = page4 >= 0 && key4 + i <= p_last;
+      for (int i = 0; i < 4; ++i) t.v_ok[half][i] = page4 >= 0 && key4 + i <= p_last;
+#pragma unroll
+      for (int xg = 0; xg < HPW / SH; ++xg) {
+        const int g = (w * HPW + xg * SH) / GS;
+        const T* k_row = k_pages + (t.k_at[half] + (long)g * page_size) * D;
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) {
+          const bool in = c * KC + VEC * quad + VEC <= D;
+          t.kv[half][xg][c] = load_or_zero<T>(k_row + (in ? c * KC + VEC * quad : 0), t.k_ok[half] && in);
+        }
+      }
     }
+  };
+
+  // The queries of the wave's heads do not change from tile to tile: they stay in registers where that takes at
+  // most 32 of them (else they are read again for every tile, through the L1 cache).
+  constexpr bool kKeepQ = HPW * KCH * (int)(sizeof(typename Atom<T>::vec_t) / 4) <= 32;
+  typename Atom<T>::vec_t qv[kKeepQ ? HPW : 1][kKeepQ ? KCH : 1];
+  if constexpr (kKeepQ) {
+#pragma unroll
+    for (int x = 0; x < HPW; ++x)
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) {
+        const bool in = c * KC + VEC * quad + VEC <= D;
+        qv[x][c] = load_or_zero<T>(q_row + (w * HPW + x) * D + (in ? c * KC + VEC * quad : 0), row_ok && in);
+      }
+  }
+
+  Ahead now;
+  if (run * per_run < step_end) request(run * per_run, now);
+  for (int step = run * per_run; step < step_end; ++step) {
+    const int tile = step < kept_tiles ? step : lo_tile + (step - kept_tiles);
+    const int key0 = tile * kTileKeys;
+    long v_at[2];
+    bool v_ok[2][4];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      v_at[half] = now.v_at[half];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v_ok[half][i] = now.v_ok[half][i];
+    }
+    // -- 1. transposed raw scores of the wave's own heads ------------------------------------
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
 #pragma unroll
       for (int xg = 0; xg < HPW / SH; ++xg) {
-        const int g = (w * HPW + xg * SH) / GS;
-        const T* k_row = k_pages + (k_at[half] + (long)g * page_size) * D;
-        typename Atom<T>::vec_t kv[KCH];
-#pragma unroll
-        for (int c = 0; c < KCH; ++c) {
-          const bool in = c * KC + VEC * quad + VEC <= D;
-          kv[c] = load_or_zero<T>(k_row + (in ? c * KC + VEC * quad : 0), k_ok[half] && in);
-        }
 #pragma unroll
         for (int xs = 0; xs < SH; ++xs) {
           const int h = w * HPW + xg * SH + xs;
           f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int c = 0; c < KCH; ++c) {
-            const bool in = c * KC + VEC * quad + VEC <= D;
-            Atom<T>::mma(s, kv[c], load_or_zero<T>(q_row + h * D + (in ? c * KC + VEC * quad : 0), row_ok && in));
+            if constexpr (kKeepQ) {
+              Atom<T>::mma(s, now.kv[half][xg][c], qv[xg * SH + xs][c]);
+            } else {
+              const bool in = c * KC + VEC * quad + VEC <= D;
+              Atom<T>::mma(s, now.kv[half][xg][c],
+                           load_or_zero<T>(q_row + h * D + (in ? c * KC + VEC * quad : 0), row_ok && in));
+            }
           }
           raw_s[h][half][lane] = f32x4{s[0] * scale, s[1] * scale, s[2] * scale, s[3] * scale};
         }
       }
     }
-    __syncthreads();
+    if (step + 1 < step_end) request(step + 1, now);  // (the products above have taken this tile's keys)
+    lds_barrier();
     // -- 2. mix, mask, online softmax ---------------------------------------------------------------
     bool see[2][4];
 #pragma unroll
@@ -175,9 +223,9 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
       for (int x = 0; x < HPW; ++x) {
         const float weight = talk_s[(w * HPW + x) * H + o];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          mixed[x][0][i] = mixed[x][0][i] + weight * r0[i];
-          mixed[x][1][i] = mixed[x][1][i] + weight * r1[i];
+        for (int i = 0; i < 4; ++i) {  // (fused multiply-adds, written as such: this loop is the kernel's vector work)
+          mixed[x][0][i] = fmaf(weight, r0[i], mixed[x][0][i]);
+          mixed[x][1][i] = fmaf(weight, r1[i], mixed[x][1][i]);
         }
       }
     }
@@ -205,6 +253,43 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
       m_run[x] = m_new;
     }
     // -- 3. values: column 16 b + l16 of V^T, keys 4 quad .. 4 quad + 3 of each half ----------------
+    // Two things are the same for every lane of most tiles and are asked of the whole wave once: whether all
+    // keys of the tile are held (then no value has to be replaced by a zero) and whether no row's maximum moved
+    // (then no accumulator has to be scaled).
+    bool held = true, moved = false;
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) held = held && v_ok[half][i];
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) moved = moved || shrink[x] != 1.0f;
+    const bool all_held = __all(held) != 0 && DV % 16 == 0;
+    const bool none_moved = __all(!moved) != 0;
+    if (!none_moved) {
+#pragma unroll
+      for (int x = 0; x < HPW; ++x)
+#pragma unroll
+        for (int b = 0; b < VB; ++b)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[x][b][i] = acc[x][b][i] * shrink[x];
+    }
+    // the weights as the second operand, once a head
+    typename Atom<T>::vec_t pb[HPW][sizeof(T) == 2 ? 1 : 2];
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) {
+      if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pb[x][0][i] = (bf16_t)mixed[x][0][i];
+          pb[x][0][4 + i] = (bf16_t)mixed[x][1][i];
+        }
+      } else {
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pb[x][half][i] = mixed[x][half][i];
+      }
+    }
 #pragma unroll
     for (int xg = 0; xg < HPW / SH; ++xg) {
       const int g = (w * HPW + xg * SH) / GS;
@@ -216,48 +301,41 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
           const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[0] + column);
           const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[1] + column);
           bf16x8 a;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            a[i] = (v_ok[0][i] && col_ok) ? v0[i] : (bf16_t)0.f;
-            a[4 + i] = (v_ok[1][i] && col_ok) ? v1[i] : (bf16_t)0.f;
-          }
-#pragma unroll
-          for (int xs = 0; xs < SH; ++xs) {
-            const int x = xg * SH + xs;
-            bf16x8 pb;
+          if (all_held) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              acc[x][b][i] = acc[x][b][i] * shrink[x];
-              pb[i] = (bf16_t)mixed[x][0][i];
-              pb[4 + i] = (bf16_t)mixed[x][1][i];
+              a[i] = v0[i];
+              a[4 + i] = v1[i];
             }
-            Atom<T>::mma(acc[x][b], a, pb);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              a[i] = (v_ok[0][i] && col_ok) ? v0[i] : (bf16_t)0.f;
+              a[4 + i] = (v_ok[1][i] && col_ok) ? v1[i] : (bf16_t)0.f;
+            }
           }
+#pragma unroll
+          for (int xs = 0; xs < SH; ++xs) Atom<T>::mma(acc[xg * SH + xs][b], a, pb[xg * SH + xs][0]);
         } else {
           f32x4 a[2];
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             const f32x4 v = *reinterpret_cast<const f32x4*>(v_pages + v_at[half] + column);
+            if (all_held) {
+              a[half] = v;
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) a[half][i] = (v_ok[half][i] && col_ok) ? v[i] : 0.f;
-          }
-#pragma unroll
-          for (int xs = 0; xs < SH; ++xs) {
-            const int x = xg * SH + xs;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[x][b][i] = acc[x][b][i] * shrink[x];
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-              f32x4 pb;
-#pragma unroll
-              for (int i = 0; i < 4; ++i) pb[i] = mixed[x][half][i];
-              Atom<T>::mma(acc[x][b], a[half], pb);
+              for (int i = 0; i < 4; ++i) a[half][i] = (v_ok[half][i] && col_ok) ? v[i] : 0.f;
             }
           }
+#pragma unroll
+          for (int xs = 0; xs < SH; ++xs)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) Atom<T>::mma(acc[xg * SH + xs][b], a[half], pb[xg * SH + xs][half]);
         }
       }
     }
-    __syncthreads();
+    lds_barrier();
   }
   if (!row_ok) return;
   if (n_runs > 1) {
