@@ -163,8 +163,9 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 // Two launches.  The first computes q, a and b of every token once, elementwise over the whole step
 // (they do not depend on the state): gates [T][H][3][dp], dp = D rounded up to a multiple of 32,
 // zeros beyond D.  The second walks the tokens: a workgroup takes (request, head, block of 16
-// columns of the state).  A wave holds 32 rows of these columns: lane (column l16 = lane / 4,
-// quarter = lane % 4) keeps the rows 32 g + 8 quarter + {0..7} of its column in registers, and the
+// columns of the state).  A wave holds 16 rows of these columns: lane (column l16 = lane / 4,
+// quarter = lane % 4) keeps the rows 16 g + 4 quarter + {0..3} of its column in registers (few rows a lane
+// and many waves: the walk is a chain of dependent instructions, and a second wave on a SIMD fills its gaps), and the
 // waves walk the request's tokens in order, sixteen at a time: their gates and values are copied to
 // LDS by all threads, every lane adds its rows' part of o_t (fused multiply-adds, written as
 // such), the four quarters of a column are neighbouring lanes and are added by exchanges inside the quad,
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 // (into registers); after the walk they are written to the other set, one barrier follows, and the
 // waves' parts of the chunk's o_t are added and stored while the next chunk is walked.
 // ---------------------------------------------------------------------------
-constexpr int kRecRows = 8;     // rows of the state a lane keeps
+constexpr int kRecRows = 4;     // rows of the state a lane keeps (a multiple of 4)
 constexpr int kRecCols = 16;    // columns of the state a workgroup takes
 constexpr int kRecWaveRows = 4 * kRecRows;  // rows a wave holds
 constexpr int kRecTokens = 16;  // tokens copied at a time
@@ -231,7 +232,7 @@ __device__ __forceinline__ float quad_sum(float v) {
   return v;
 }
 
-__global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ gates, const float* __restrict__ raw,
+__global__ __launch_bounds__(1024) void linrec_kernel(const float* __restrict__ gates, const float* __restrict__ raw,
                                                      long ld, int v_at, int H, int D, int DV,
                                                      const SeqMeta* __restrict__ seqs, float* __restrict__ state,
                                                      float* __restrict__ out, long ldo) {
@@ -298,9 +299,9 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
   auto walk_chunk = [&](float* base, int n) LS_INLINED {
     const float* v_s = base + kRecTokens * token;
     float* o_s = base + kRecTokens * token + kRecTokens * kRecCols;  // [waves][tokens][columns]
-    // a token's operands: eight q, a and b of the lane's rows (two vectors each) and its column's value
+    // a token's operands: q, a and b of the lane's rows and its column's value
     struct Operands {
-      f32x4 q[2], a[2], b[2];
+      f32x4 q[kRecRows / 4], a[kRecRows / 4], b[kRecRows / 4];
       float v;
     };
     auto fetch = [&](int tt) LS_INLINED {
@@ -308,7 +309,7 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
       const float* qa = base + tt * token + row0;
       x.v = v_s[tt * kRecCols + l16];
 #pragma unroll
-      for (int k = 0; k < 2; ++k) {
+      for (int k = 0; k < kRecRows / 4; ++k) {
         x.q[k] = *reinterpret_cast<const f32x4*>(qa + 4 * k);
         x.a[k] = *reinterpret_cast<const f32x4*>(qa + dp + 4 * k);
         x.b[k] = *reinterpret_cast<const f32x4*>(qa + 2 * dp + 4 * k);
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(512) void linrec_kernel(const float* __restrict__ g
         S[r] = fmaf(x.a[r >> 2][r & 3], S[r], x.b[r >> 2][r & 3] * x.v);
         o = fmaf(S[r], x.q[r >> 2][r & 3], o);
       }
-      o = quad_sum(o);  // the four quarters of the wave: rows 8 quarter .. of the same column
+      o = quad_sum(o);  // the four quarters of the wave: rows kRecRows * quarter .. of the same column
       if (quarter == 0) o_s[(g * kRecTokens + tt) * kRecCols + l16] = o;
     };
     if (n == kRecTokens) {
@@ -482,7 +483,7 @@ extern "C" int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, i
   return check_launch("talk_qkv");
 }
 
-extern "C" int ls_linrec_max_dim() { return 8 * kRecWaveRows; }
+extern "C" int ls_linrec_max_dim() { return 16 * kRecWaveRows; }
 
 extern "C" long ls_linrec_gate_floats(int n_tokens, int H, int D) {
   const int dp = (D + kRecWaveRows - 1) / kRecWaveRows * kRecWaveRows;

@@ -371,7 +371,7 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
 
 // Fold the runs of row blocks: a fold item (first work item, runs, first packed row, rows) names the work items
 // first .. first + runs - 1 of one row block, whose partial results are folded in ascending order for each of its
-// rows.  One workgroup a (fold item, head).
+// rows.  One workgroup a (fold item, head, row).
 template <typename T>
 __global__ __launch_bounds__(64) void talk_combine_kernel(const float* __restrict__ part, int part_rows,
                                                           const int* __restrict__ folds, T* __restrict__ out,
@@ -380,7 +380,7 @@ __global__ __launch_bounds__(64) void talk_combine_kernel(const float* __restric
   const int row0 = folds[4 * blockIdx.x + 2], rows = folds[4 * blockIdx.x + 3];
   const int h = blockIdx.y;
   const long stride = (long)part_rows * H * (DV + 2);  // from a run to the next
-  for (int r = 0; r < rows; ++r) {
+  for (int r = blockIdx.z; r < rows; r += gridDim.z) {
     const float* mine = part + (((long)first * part_rows + r) * H + h) * (DV + 2);
     float top = kNegSentinel;
     for (int k = 0; k < n_runs; ++k) top = fmaxf(top, mine[k * stride + DV]);
@@ -433,7 +433,7 @@ extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void*
                        (const float*)k_pages, (const float*)v_pages, page_size, table, table_stride,
                        (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (float*)out, ldo, part, part_rows);
     if (n_folds > 0)
-      hipLaunchKernelGGL(talk_combine_kernel<float>, dim3(n_folds, H), dim3(64), 0, s, part, part_rows, folds,
+      hipLaunchKernelGGL(talk_combine_kernel<float>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows, folds,
                          (float*)out, ldo);
   } else if (dtype == kBF16) {
     LS_REQUIRE(ldq % 8 == 0, "talk_attention: query rows must be 16-byte aligned");
@@ -442,7 +442,7 @@ extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void*
                        (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (bf16_t*)out, ldo, part,
                        part_rows);
     if (n_folds > 0)
-      hipLaunchKernelGGL(talk_combine_kernel<bf16_t>, dim3(n_folds, H), dim3(64), 0, s, part, part_rows, folds,
+      hipLaunchKernelGGL(talk_combine_kernel<bf16_t>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows, folds,
                          (bf16_t*)out, ldo);
   } else {
     return fail("talk_attention: unknown dtype %d", dtype);

@@ -32,6 +32,7 @@ ROWS_A_BLOCK = 16      # query rows of a work item of the attention kernel
 TILE_KEYS = 32         # keys of a tile of the attention kernel
 MAX_RUNS = 16          # the most runs the keys of a row block are dealt to
 TILES_A_RUN = 8        # a row block of a prompt portion is cut into runs of at least this many tiles
+TILES_A_DECODE_RUN = int(__import__("os").environ.get("LOCKSTEP_TALK_DECODE_TILES", "2"))   # ... of a decoded token
 
 
 @register_part("talking_attention")
@@ -129,7 +130,7 @@ class TalkingAttention(Mixer):
             # two above the longest context only)
             longest = min(int(ctx.kv_len.max()) + ctx.horizon, self.window + self.keep_first)
             tiles = 1 << max(0, (-(-longest // TILE_KEYS) - 1).bit_length())
-            runs = max(1, min(MAX_RUNS, (2 * cus) // ctx.n_seqs, tiles // 4))
+            runs = max(1, min(MAX_RUNS, (2 * cus) // ctx.n_seqs, tiles // TILES_A_DECODE_RUN))
             seq = np.repeat(np.arange(ctx.n_seqs), runs)
             items = np.stack([seq, np.zeros_like(seq), np.tile(np.arange(runs), ctx.n_seqs), np.full_like(seq, runs)], axis=1)
             rows = np.arange(ctx.n_seqs)            # a request's one row is packed row i
