@@ -168,7 +168,7 @@ class CacheManager:
         for unit, spec in enumerate(unit_specs):
             if isinstance(spec, PagedKVSpec):
                 keyed.setdefault((spec.num_kv_heads, spec.head_dim, spec.window, spec.value_dim,
-                                  int(spec.keep_first or 0)), []).append(unit)
+                                  int(spec.keep_first or 0), spec.chunk), []).append(unit)
             elif isinstance(spec, StateSpec):
                 self.state_units[unit] = spec
             elif spec is not None:
@@ -178,8 +178,8 @@ class CacheManager:
             raise ValueError(f"{len(keyed)} cache groups but {len(sizes)} pool sizes")
         self.groups: list[CacheGroup] = []
         self.unit_place: dict[int, tuple[int, int]] = {}
-        for index, ((h, d, window, value_dim, keep_first), units) in enumerate(keyed.items()):
-            group = CacheGroup(index, PagedKVSpec(h, d, window, value_dim, keep_first), units, sizes[index], page_size, max_requests,
+        for index, ((h, d, window, value_dim, keep_first, chunk), units) in enumerate(keyed.items()):
+            group = CacheGroup(index, PagedKVSpec(h, d, window, value_dim, keep_first, chunk), units, sizes[index], page_size, max_requests,
                                self.max_pages_per_request, torch_dtype, device)
             self.groups.append(group)
             for position, unit in enumerate(units):
@@ -224,9 +224,12 @@ class CacheManager:
 
     def _first_needed(self, group: CacheGroup, next_position: int) -> int:
         """Logical page below which a query at ``next_position`` reads nothing."""
-        if group.spec.window is None:
-            return 0
-        return max(0, next_position - group.spec.window + 1) // self.page_size
+        first = 0
+        if group.spec.window is not None:
+            first = max(first, next_position - group.spec.window + 1)
+        if group.spec.chunk:
+            first = max(first, next_position // group.spec.chunk * group.spec.chunk)
+        return first // self.page_size
 
     def _kept_pages(self, group: CacheGroup) -> int:
         """Logical pages at the start of a request that a window never releases (they hold the
@@ -342,6 +345,8 @@ class CacheManager:
             return f"the layers' caches form {len(self.groups)} groups with page tables of their own"
         if self.groups[0].spec.window is not None:
             return "the layers keep a window of keys only, so early pages of a prefix are gone"
+        if self.groups[0].spec.chunk:
+            return "the layers keep the keys of the current chunk only, so early pages of a prefix are gone"
         return None
 
     def adopt(self, request_id: Hashable, pages: Sequence[int]) -> None:

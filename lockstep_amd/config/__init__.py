@@ -7,9 +7,10 @@ from .registry import (config_class_for, config_from_dict, config_from_dir,
                        unregister_architecture)
 from .qwen3 import Qwen3Config
 from .bikovik import BikovikConfig
+from .biberax import BiberaxConfig
 
 __all__ = [
     "ConfigError", "LayerSpec", "ModelConfig", "ModelSpec", "PartSpec", "ScheduleEntry",
     "config_class_for", "config_from_dict", "config_from_dir", "known_architectures",
-    "register_architecture", "unregister_architecture", "Qwen3Config", "BikovikConfig",
+    "register_architecture", "unregister_architecture", "Qwen3Config", "BikovikConfig", "BiberaxConfig",
 ]

@@ -1,0 +1,299 @@
+// A feed-forward of many small experts of which each token uses a few (routing on the device, no
+// word of it read by the host):
+//
+//   z[t]        = router logits of token t (float, computed by the caller's matrix product) + bias
+//   chosen(t)   = the `top` experts with the largest z[t] (the lower index wins a tie), in that order
+//   w[t, k]     = softmax over the chosen logits alone
+//   expert e    : y = act(W_gate[e] x, W_up[e] x),  out = W_down[e] y
+//                 act(g, u) = g' sigmoid(alpha g') (u' + 1),  g' = min(g, limit),  u' = clamp(u, -limit, limit)
+//   P[k][t]     = w[t, k] * expert chosen(t)[k] (x[t])        (float; the caller adds the slices in order)
+//
+// Four launches.  (1) route: one thread a token picks the experts and their weights.  (2) group: the
+// (token, choice) pairs are put in the order of their experts (a stable counting sort by one workgroup:
+// a wave an expert counts its pairs by ballots, then places them), and every expert's pairs are cut
+// into tiles of ROWS rows; the tile list has a fixed capacity that depends on the sizes only, unused
+// tiles are marked.  (3) the gate and up products of every tile with the activation as epilogue; (4)
+// the down products, scaled and scattered to P.  Products use the 16x16 MFMA atom with the weight
+// rows as first operand (a lane ends with four consecutive output columns of one row); a row's
+// contraction is one chain over ascending K from zero, so its bits do not depend on the tile it is in
+// or on what else is in the step.  A weight fragment is loaded once and multiplied with all RT row
+// tiles of a wave.
+
+#include "common.h"
+
+namespace ls {
+
+constexpr int kMaxTop = 16;
+
+__device__ __forceinline__ float sigmoid_e(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// ---------------------------------------------------------------------------
+// (1) One thread a token: expert [T][top] int, weight [T][top] float.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ z, long ldz,
+                                                         const float* __restrict__ bias, int n_tokens, int E, int top,
+                                                         int* expert, float* weight) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= n_tokens) return;
+  const float* row = z + (long)t * ldz;
+  // (the picks so far are kept in the outputs themselves: a thread reads back what it wrote)
+  int* picked = expert + (long)t * top;
+  float* value = weight + (long)t * top;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float best_v = 0.f;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken = taken || picked[j] == e;
+      if (taken) continue;
+      const float v = row[e] + (bias ? bias[e] : 0.f);
+      if (best < 0 || v > best_v) {
+        best = e;
+        best_v = v;
+      }
+    }
+    picked[k] = best;
+    value[k] = best_v;
+  }
+  const float largest = value[0];
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const float ex = expf(value[k] - largest);
+    value[k] = ex;
+    sum = sum + ex;
+  }
+  for (int k = 0; k < top; ++k) value[k] = value[k] / sum;
+}
+
+// ---------------------------------------------------------------------------
+// (2) One workgroup of 16 waves.  order [P]: the pairs (token * top + choice) sorted by expert, stable.
+// tiles [cap][4]: expert (-1: unused), first place in order, rows, 0.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void route_group_kernel(const int* __restrict__ expert, int P, int E, int rows_a_tile,
+                                                           int* __restrict__ order, int* __restrict__ tiles, int cap,
+                                                           int* __restrict__ counts) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  // counts [E] (pairs of an expert), then their running sums; in global scratch: E has no bound here
+  for (int e = w; e < E; e += 16) {
+    int n = 0;
+    for (int p0 = 0; p0 < P; p0 += 64) {
+      const bool mine = p0 + lane < P && expert[p0 + lane] == e;
+      n += __popcll(__ballot(mine));
+    }
+    if (lane == 0) counts[e] = n;
+  }
+  __syncthreads();
+  for (int e = w; e < E; e += 16) {
+    int base = 0, tile = 0;
+    for (int j = 0; j < e; ++j) {      // (every lane the same few additions)
+      base += counts[j];
+      tile += (counts[j] + rows_a_tile - 1) / rows_a_tile;
+    }
+    const int n = counts[e];
+    for (int i = lane; i * rows_a_tile < n; i += 64) {
+      if (tile + i < cap) {
+        tiles[4 * (tile + i)] = e;
+        tiles[4 * (tile + i) + 1] = base + i * rows_a_tile;
+        tiles[4 * (tile + i) + 2] = min(rows_a_tile, n - i * rows_a_tile);
+        tiles[4 * (tile + i) + 3] = 0;
+      }
+    }
+    if (e == E - 1) {
+      const int used = tile + (n + rows_a_tile - 1) / rows_a_tile;
+      for (int i = used + lane; i < cap; i += 64) {
+        tiles[4 * i] = -1;
+        tiles[4 * i + 1] = tiles[4 * i + 2] = tiles[4 * i + 3] = 0;
+      }
+    }
+    int at = base;
+    for (int p0 = 0; p0 < P; p0 += 64) {
+      const bool mine = p0 + lane < P && expert[p0 + lane] == e;
+      const unsigned long long votes = __ballot(mine);
+      if (mine) order[at + __popcll(votes & ((1ull << lane) - 1ull))] = p0 + lane;
+      at += __popcll(votes);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// (3) act [P][ldy] (T) = act(x[token] W_gate[e]^T, x[token] W_up[e]^T) for the pairs of every tile, in the
+// order of `order`.  w_gate, w_up [E][F][K].  A workgroup: one tile, four waves with 16 columns of F each.
+// ---------------------------------------------------------------------------
+template <typename T, int RT>
+__global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restrict__ x, long ldx,
+                                                              const T* __restrict__ w_gate, const T* __restrict__ w_up,
+                                                              int F, int K, int top, const int* __restrict__ order,
+                                                              const int* __restrict__ tiles, float limit, float alpha,
+                                                              T* __restrict__ act, long ldy) {
+  constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
+  const int e = tiles[4 * blockIdx.x];
+  if (e < 0) return;
+  const int first = tiles[4 * blockIdx.x + 1], rows = tiles[4 * blockIdx.x + 2];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4;
+  const int col0 = (blockIdx.y * 4 + w) * 16;
+  if (col0 >= F) return;
+  const bool w_ok = col0 + l16 < F;
+  const T* g_row = w_gate + ((long)e * F + (w_ok ? col0 + l16 : 0)) * K;
+  const T* u_row = w_up + ((long)e * F + (w_ok ? col0 + l16 : 0)) * K;
+  const T* x_row[RT];
+  bool x_ok[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    x_ok[r] = 16 * r + l16 < rows;
+    const int pair = x_ok[r] ? order[first + 16 * r + l16] : 0;
+    x_row[r] = x + (long)(pair / top) * ldx;
+  }
+  f32x4 acc_g[RT], acc_u[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc_g[r] = acc_u[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool aligned = K % VEC == 0;
+  for (int k0 = 0; k0 < K; k0 += KC) {
+    const int k = k0 + VEC * quad;
+    const typename Atom<T>::vec_t a_g = load_vec<T>(g_row, 0, k, K, 0, w_ok, aligned);
+    const typename Atom<T>::vec_t a_u = load_vec<T>(u_row, 0, k, K, 0, w_ok, aligned);
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      const typename Atom<T>::vec_t b = load_vec<T>(x_row[r], 0, k, K, 0, x_ok[r], aligned);
+      Atom<T>::mma(acc_g[r], a_g, b);
+      Atom<T>::mma(acc_u[r], a_u, b);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    if (!x_ok[r]) continue;
+    T* dst = act + (long)(first + 16 * r + l16) * ldy;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = col0 + 4 * quad + i;
+      if (c < F) {
+        const float g = fminf(acc_g[r][i], limit);
+        const float u = fminf(fmaxf(acc_u[r][i], -limit), limit);
+        dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + 1.0f));
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// (4) P[choice][token][:] = weight[pair] * (act[place] W_down[e]^T).  w_down [E][N][F]; P [top][n_tokens][N] float.
+// ---------------------------------------------------------------------------
+template <typename T, int RT>
+__global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__ act, long ldy,
+                                                           const T* __restrict__ w_down, int N, int F, int top,
+                                                           int n_tokens, const int* __restrict__ order,
+                                                           const int* __restrict__ tiles,
+                                                           const float* __restrict__ weight, float* __restrict__ P) {
+  constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
+  const int e = tiles[4 * blockIdx.x];
+  if (e < 0) return;
+  const int first = tiles[4 * blockIdx.x + 1], rows = tiles[4 * blockIdx.x + 2];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4;
+  const int col0 = (blockIdx.y * 4 + w) * 16;
+  if (col0 >= N) return;
+  const bool w_ok = col0 + l16 < N;
+  const T* d_row = w_down + ((long)e * N + (w_ok ? col0 + l16 : 0)) * F;
+  const T* y_row[RT];
+  bool y_ok[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    y_ok[r] = 16 * r + l16 < rows;
+    y_row[r] = act + (long)(first + (y_ok[r] ? 16 * r + l16 : 0)) * ldy;
+  }
+  f32x4 acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool aligned = F % VEC == 0 && ldy % VEC == 0;
+  for (int k0 = 0; k0 < F; k0 += KC) {
+    const int k = k0 + VEC * quad;
+    const typename Atom<T>::vec_t a = load_vec<T>(d_row, 0, k, F, 0, w_ok, aligned);
+#pragma unroll
+    for (int r = 0; r < RT; ++r) Atom<T>::mma(acc[r], a, load_vec<T>(y_row[r], 0, k, F, 0, y_ok[r], aligned));
+  }
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    if (!y_ok[r]) continue;
+    const int pair = order[first + 16 * r + l16];
+    const float share = weight[pair];
+    float* dst = P + ((long)(pair % top) * n_tokens + pair / top) * N;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = col0 + 4 * quad + i;
+      if (c < N) dst[c] = share * acc[r][i];
+    }
+  }
+}
+
+}  // namespace ls
+
+LS_DEFINE_ERROR_API
+
+using namespace ls;
+
+extern "C" int ls_experts_max_top() { return kMaxTop; }
+
+// Tiles that the pairs of n_tokens tokens can need at most, with rows_a_tile rows each.
+extern "C" int ls_experts_tile_capacity(int n_tokens, int E, int top, int rows_a_tile) {
+  const long pairs = (long)n_tokens * top;
+  return (int)(pairs / rows_a_tile + (pairs < E ? pairs : E));
+}
+
+// z [n_tokens][ldz] float router logits, bias [E] or null -> expert, weight [n_tokens][top]; order [n_tokens * top];
+// tiles [cap][4]; counts: scratch of E ints.  rows_a_tile 16, 32 or 64.
+extern "C" int ls_experts_route(const float* z, long ldz, const float* bias, int n_tokens, int E, int top,
+                                int rows_a_tile, int* expert, float* weight, int* order, int* tiles, int cap,
+                                int* counts, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && E > 0 && top > 0 && top <= E && top <= kMaxTop && ldz >= E,
+             "experts_route: %d tokens, %d experts, %d chosen (at most %d)", n_tokens, E, top, kMaxTop);
+  LS_REQUIRE(rows_a_tile == 16 || rows_a_tile == 32 || rows_a_tile == 64, "experts_route: tiles of %d rows", rows_a_tile);
+  LS_REQUIRE(z && expert && weight && order && tiles && counts, "experts_route: null operand");
+  LS_REQUIRE(cap >= ls_experts_tile_capacity(n_tokens, E, top, rows_a_tile), "experts_route: %d tiles are too few", cap);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 255) / 256), dim3(256), 0, s, z, ldz, bias, n_tokens, E, top,
+                     expert, weight);
+  hipLaunchKernelGGL(route_group_kernel, dim3(1), dim3(1024), 0, s, expert, n_tokens * top, E, rows_a_tile, order, tiles,
+                     cap, counts);
+  return check_launch("experts_route");
+}
+
+// x [n_tokens][ldx]; w_gate, w_up [E][F][K]; w_down [E][N][F]; act: scratch [n_tokens * top][ldy] of the compute
+// dtype; P [top][n_tokens][N] float.
+extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* w_gate, const void* w_up,
+                                const void* w_down, int n_tokens, int E, int top, int K, int F, int N,
+                                int rows_a_tile, const int* order, const int* tiles, int cap, const float* weight,
+                                float limit, float alpha, void* act, long ldy, float* P, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && E > 0 && top > 0 && K > 0 && F > 0 && N > 0 && ldx >= K && ldy >= F, "experts_apply: bad sizes");
+  LS_REQUIRE(rows_a_tile == 16 || rows_a_tile == 32 || rows_a_tile == 64, "experts_apply: tiles of %d rows", rows_a_tile);
+  LS_REQUIRE(x && w_gate && w_up && w_down && order && tiles && weight && act && P && cap > 0, "experts_apply: null operand");
+  LS_REQUIRE(limit > 0.f, "experts_apply: the limit must be positive");
+  LS_REQUIRE(dtype == kF32 || dtype == kBF16, "experts_apply: unknown dtype %d", dtype);
+  const int vec = dtype == kF32 ? 4 : 8;
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(act) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(w_gate) % 16 == 0 && reinterpret_cast<uintptr_t>(w_up) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(w_down) % 16 == 0 && (K % vec != 0 || ldx % vec == 0),
+             "experts_apply: operands must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid_up(cap, (F + 63) / 64), grid_down(cap, (N + 63) / 64);
+#define LS_EXPERTS(T_, RT_)                                                                                           \
+  do {                                                                                                                \
+    hipLaunchKernelGGL((experts_gate_up_kernel<T_, RT_>), grid_up, dim3(256), 0, s, (const T_*)x, ldx,                \
+                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, (T_*)act, ldy);     \
+    hipLaunchKernelGGL((experts_down_kernel<T_, RT_>), grid_down, dim3(256), 0, s, (const T_*)act, ldy,               \
+                       (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
+  } while (0)
+#define LS_EXPERTS_BY_ROWS(T_)                 \
+  switch (rows_a_tile) {                       \
+    case 16: LS_EXPERTS(T_, 1); break;         \
+    case 32: LS_EXPERTS(T_, 2); break;         \
+    default: LS_EXPERTS(T_, 4); break;         \
+  }
+  if (dtype == kF32) {
+    LS_EXPERTS_BY_ROWS(float)
+  } else {
+    LS_EXPERTS_BY_ROWS(bf16_t)
+  }
+#undef LS_EXPERTS_BY_ROWS
+#undef LS_EXPERTS
+  return check_launch("experts_apply");
+}

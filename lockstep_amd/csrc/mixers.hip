@@ -1,7 +1,8 @@
 // Kernels of the mixers, norms and activations beyond the softmax-attention decoder: Dynamic Tanh
 // norm (with the deferred residual addition), the clamped gated unit, the soft cap of the logits,
 // the post pass of an attention projection with biases, partial rotation, value mixing and cache
-// write for keys and values of different sizes, the linear recurrence with per-row decay and write
+// write for keys and values of different sizes (and its sibling with a norm over the whole projection,
+// rotation of neighbouring pairs and keys that are the values), the linear recurrence with per-row decay and write
 // gates (HGRN2, retention), and the per-head RMS norm with an optional weight and gate.
 //
 // Everything here is computed in float whatever the compute dtype T is: T is the type of what a
@@ -151,6 +152,97 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
   }
   const int g = c / DV, i = c % DV;
   if (page >= 0) v_pages[(((long)page * G + g) * DV + i) * page_size + slot] = from_f32<T>(own);
+}
+
+// ---------------------------------------------------------------------------
+// Post pass of an attention projection raw [T][ld] float = q (H heads of D) | k (G of D) | v (G of DV, absent
+// when the keys are the values) | whatever follows (an output gate, which this pass leaves alone):
+//   biases added (bias [H*D + G*D (+ G*DV)] or null);
+//   v = k as projected, with its bias, before any norm (keys_are_values; DV == D);
+//   q and k each divided by the root mean square over ALL their heads at once (the whole projection is one
+//   vector: x / sqrt(mean(x^2) + eps)), times a weight an element (q_norm [H*D], k_norm [G*D]; null: no norm);
+//   q and k rotated on their first `rot` dimensions at the token's position, pairs (i, i + rot/2) or, with
+//   `neighbours`, (2i, 2i + 1), angle tables [positions][rot/2];
+//   q -> q_out [T][H*D] (T);  k -> key pages [page][G][slot][D];  v -> value pages [page][G][DV][slot].
+// One workgroup a token.  The sums of squares: thread t adds the squares of elements t, t + 256, ... in
+// ascending order, then a butterfly over the wave and the wave sums in wave order: a function of the sizes only.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float block_sum256(float v, float* scratch) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) scratch[w] = v;
+  __syncthreads();
+  return ((scratch[0] + scratch[1]) + scratch[2]) + scratch[3];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_post_kernel(
+    const float* __restrict__ raw, long ld, int H, int G, int D, int DV, int keys_are_values,
+    const float* __restrict__ bias, const float* __restrict__ q_norm, const float* __restrict__ k_norm, float eps,
+    const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot, int neighbours,
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, const SeqMeta* __restrict__ seqs,
+    const int* __restrict__ table, int table_stride, T* __restrict__ q_out, long ldq, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int page_size) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const float* row = raw + (long)t * ld;
+  const int pos = tok_pos[t];
+  const int nq = H * D, nk = G * D, nv = G * DV;
+  float rq = 1.0f, rk = 1.0f;
+  if (q_norm) {
+    float part = 0.f;
+    for (int e = threadIdx.x; e < nq; e += 256) {
+      const float x = row[e] + (bias ? bias[e] : 0.f);
+      part = part + x * x;
+    }
+    rq = 1.0f / sqrtf(block_sum256(part, scratch) / (float)nq + eps);
+  }
+  if (k_norm) {
+    float part = 0.f;
+    for (int e = threadIdx.x; e < nk; e += 256) {
+      const float x = row[nq + e] + (bias ? bias[nq + e] : 0.f);
+      part = part + x * x;
+    }
+    rk = 1.0f / sqrtf(block_sum256(part, scratch) / (float)nk + eps);
+  }
+  const int table_row = seqs[tok_seq[t]].table_row;
+  const int page = table[(long)table_row * table_stride + pos / page_size];
+  const int slot = pos % page_size;
+  const int half = rot >> 1;
+  const float* cos_row = cos_table + (long)pos * half;
+  const float* sin_row = sin_table + (long)pos * half;
+  // element e of q | k as the attention reads it: bias, norm, rotation
+  auto finished = [&](int e) LS_INLINED {
+    const bool is_q = e < nq;
+    const float* w = is_q ? q_norm : k_norm;
+    const int at = is_q ? e : e - nq;      // index into the norm weight
+    const float r = is_q ? rq : rk;
+    float own = row[e] + (bias ? bias[e] : 0.f);
+    if (w) own = own * r * w[at];
+    const int i = e % D;
+    if (i < rot) {
+      const int pe = neighbours ? (e ^ 1) : (i < half ? e + half : e - half);
+      float other = row[pe] + (bias ? bias[pe] : 0.f);
+      if (w) other = other * r * w[is_q ? pe : pe - nq];
+      const int pair = neighbours ? (i >> 1) : (i < half ? i : i - half);
+      const bool lower = neighbours ? (i & 1) == 0 : i < half;
+      own = lower ? own * cos_row[pair] - other * sin_row[pair] : own * cos_row[pair] + other * sin_row[pair];
+    }
+    return own;
+  };
+  for (int e = threadIdx.x; e < nq; e += 256) q_out[(long)t * ldq + e] = from_f32<T>(finished(e));
+  if (page < 0) return;
+  for (int e = threadIdx.x; e < nk; e += 256) {
+    const int g = e / D, i = e % D;
+    k_pages[(((long)page * G + g) * page_size + slot) * D + i] = from_f32<T>(finished(nq + e));
+  }
+  for (int c = threadIdx.x; c < nv; c += 256) {
+    const int from = keys_are_values ? nq + c : nq + nk + c;
+    const float v = row[from] + (bias ? bias[from] : 0.f);
+    const int g = c / DV, i = c % DV;
+    v_pages[(((long)page * G + g) * DV + i) * page_size + slot] = from_f32<T>(v);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -481,6 +573,38 @@ extern "C" int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, i
     return fail("talk_qkv: unknown dtype %d", dtype);
 #undef LS_TALK_QKV
   return check_launch("talk_qkv");
+}
+
+extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int DV,
+                           int keys_are_values, const float* bias, const float* q_norm, const float* k_norm, float eps,
+                           const float* cos_table, const float* sin_table, int rot, int neighbours,
+                           int table_positions, int max_pos, const int* tok_seq, const int* tok_pos, const void* seqs,
+                           const int* table, int table_stride, void* q_out, long ldq, void* k_pages, void* v_pages,
+                           int page_size, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && H > 0 && G > 0 && D > 0 && DV > 0 && H % G == 0, "qkv_post: bad head sizes");
+  LS_REQUIRE(!keys_are_values || DV == D, "qkv_post: keys of %d elements cannot be values of %d", D, DV);
+  const long width = (long)H * D + (long)G * D + (keys_are_values ? 0 : (long)G * DV);
+  LS_REQUIRE(ld >= width && ldq >= (long)H * D && raw && q_out && k_pages && v_pages && table && seqs && tok_seq &&
+                 tok_pos && page_size > 0 && table_stride > 0,
+             "qkv_post: bad operands");
+  LS_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "qkv_post: %d rotated dimensions of %d", rot, D);
+  LS_REQUIRE(rot == 0 || (cos_table && sin_table && max_pos < table_positions),
+             "qkv_post: position %d is beyond the rotation tables (%d)", max_pos, table_positions);
+  LS_REQUIRE(max_pos / page_size < table_stride, "qkv_post: position %d is beyond the block table", max_pos);
+  LS_REQUIRE((q_norm == nullptr) == (k_norm == nullptr) && (!q_norm || eps > 0.f), "qkv_post: bad norm");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define LS_QKV_POST(T_)                                                                                               \
+  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens), dim3(256), 0, s, raw, ld, H, G, D, DV, keys_are_values,     \
+                     bias, q_norm, k_norm, eps, cos_table, sin_table, rot, neighbours, tok_seq, tok_pos,              \
+                     (const SeqMeta*)seqs, table, table_stride, (T_*)q_out, ldq, (T_*)k_pages, (T_*)v_pages, page_size)
+  if (dtype == kF32)
+    LS_QKV_POST(float);
+  else if (dtype == kBF16)
+    LS_QKV_POST(bf16_t);
+  else
+    return fail("qkv_post: unknown dtype %d", dtype);
+#undef LS_QKV_POST
+  return check_launch("qkv_post");
 }
 
 extern "C" int ls_linrec_max_dim() { return 16 * kRecWaveRows; }

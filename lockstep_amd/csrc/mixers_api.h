@@ -30,6 +30,15 @@ int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, int H, int G
                 void* q_out, long ldq, void* k_pages, void* v_pages, int page_size, int vmix_mode, const float* vmix,
                 float* v_first, long ldv, void* stream);
 
+// Post pass of an attention projection raw = q | k | v (| more): biases, a root-mean-square norm over the whole of q
+// and of k (weights q_norm [H*D], k_norm [G*D], or null), rotation in pairs (i, i + rot/2) or of neighbours, keys
+// that are also the values (keys_are_values: no v in raw, the biased unnormalised k is stored as v).
+int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int DV, int keys_are_values,
+                const float* bias, const float* q_norm, const float* k_norm, float eps, const float* cos_table,
+                const float* sin_table, int rot, int neighbours, int table_positions, int max_pos, const int* tok_seq,
+                const int* tok_pos, const void* seqs, const int* table, int table_stride, void* q_out, long ldq,
+                void* k_pages, void* v_pages, int page_size, void* stream);
+
 // Linear recurrence S_t = diag(a_t) S_(t-1) + b_t v_t^T, o_t = S_t^T q_t over the tokens of every request of the
 // step, state [slots][H][D][DV] float (mode 0: HGRN2 gates from p0 = lower bounds [H*D] and p1 = gate bias or null;
 // mode 1: retention with p0 = decay [H] and rotated q, k at the positions tok_pos [n_tokens]).  out [T][ldo] float

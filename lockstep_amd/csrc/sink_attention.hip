@@ -1,0 +1,447 @@
+// Grouped-query attention over the paged cache whose softmax has a sink, with a choice of what a query
+// sees and of what is added to its scores:
+//
+//   s_h[i, j]    = (q_h[i] . k_kv(h)[j]) * scale + bias_h[min(i - j, n_dist - 1)]   (bias optional)
+//   visible(i,j) = lo(i) <= j <= i,   lo(i) = max(window ? i - window + 1 : 0, chunk ? floor(i / chunk) chunk : 0)
+//   p_h[i, j]    = exp(s_h[i, j]) / (exp(sink_h) + sum over visible j' of exp(s_h[i, j']))  (without a sink: no term)
+//   o_h[i]       = gate_h[i] * sum_j p_h[i, j] v_kv(h)[j],   gate = sigmoid(g_h[i]) elementwise (optional)
+//
+// i and j are absolute positions; the sink is a score that has no key and no value, so the weights of a
+// row add up to less than one.  The bias is a table by distance, one row a head, whose last entry serves
+// every larger distance.
+//
+// The library is compiled for one key size LS_SA_DIM and one value size LS_SA_VDIM.  A wave owns 16 RT
+// rows of the 16x16 MFMA atom and walks the visible keys in tiles of 32 anchored at absolute positions.
+// Keys are the first operand of the score product (S^T = K Q^T: a lane ends with four consecutive keys of
+// one query row, which is how the weights enter the value product) and value columns the first operand of
+// O^T += V^T P^T (the lane that holds a row's statistics also holds its accumulators).  A key or value
+// fragment is loaded once and multiplied with all RT row tiles.  Two shapes of work:
+//   prompt portions  a workgroup takes (request, block of 16 RT rows, key/value head); its waves are the
+//                    query heads that read this key/value head, so their loads of K and V meet in the
+//                    CU's cache;
+//   decoded tokens   a wave takes (request, key/value head) and the MFMA rows are the query heads of the
+//                    group (up to 16 a wave).
+// The tiles of a row block are dealt to several work items in contiguous runs where that fills the GPU;
+// each leaves (unnormalised output, max, sum) of its run for every row and a second kernel folds the
+// runs in ascending order, adds the sink and applies the gate.
+// Scores, weights, statistics and accumulators are float; products read the compute dtype T.  Keys a
+// request does not hold (beyond its length, pages that a window or a chunk's end has released) enter as
+// zeros and are masked; their values are replaced by zeros before the product.
+
+#include "common.h"
+
+#ifndef LS_SA_DIM
+#error "compile with -DLS_SA_DIM and -DLS_SA_VDIM"
+#endif
+
+namespace ls {
+
+constexpr int D = LS_SA_DIM, DV = LS_SA_VDIM;
+static_assert(D % 8 == 0 && D <= 256, "key size must be a multiple of 8 up to 256");
+static_assert(DV % 4 == 0 && DV <= 256, "value size must be a multiple of 4 up to 256");
+constexpr int VB = (DV + 15) / 16;  // blocks of 16 value columns (the last may be partial)
+constexpr int kTileKeys = 32;
+constexpr int kMaxWaves = 4;        // query heads of a key/value head that share a workgroup
+
+struct SeqMeta {
+  int q_off, q_len, q_start, kv_len, table_row, reserved[3];
+};
+
+template <typename T>
+__device__ __forceinline__ typename Atom<T>::vec_t load_or_zero(const T* p, bool ok) {
+  typedef typename Atom<T>::vec_t vec_t;
+  // (an address that is always valid, the value chosen afterwards: the loads of a tile can be in flight together)
+  vec_t v = *reinterpret_cast<const vec_t*>(p);
+  return ok ? v : Atom<T>::zero();
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// First key that a query at position p sees.
+__device__ __forceinline__ int first_seen(int p, int window, int chunk) {
+  int lo = 0;
+  if (window > 0) lo = max(lo, p - window + 1);
+  if (chunk > 0) lo = max(lo, p / chunk * chunk);
+  return lo;
+}
+
+// DEC: a step of single decoded tokens (the rows of a tile are the heads of a key/value group).
+template <typename T, int RT, bool DEC>
+__global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
+    const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ items,
+    int H, int G, float scale, int window, int chunk, const float* __restrict__ sink,
+    const float* __restrict__ dist_bias, int n_dist, const float* __restrict__ gate, long ldg, T* __restrict__ out,
+    long ldo, float* __restrict__ part, int part_rows) {
+  constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
+  constexpr int KCH = (D + KC - 1) / KC;  // chunks of a key (lanes beyond D in the last one bring zeros)
+  constexpr int ROWS = 16 * RT;
+  // a work item: request of the step, block of ROWS of its rows, which run of the tiles, of how many runs
+  const int seq = items[4 * blockIdx.x], rb = items[4 * blockIdx.x + 1];
+  const int run = items[4 * blockIdx.x + 2], n_runs = max(1, items[4 * blockIdx.x + 3]);
+  const SeqMeta m = seqs[seq];
+  const int GS = H / G, g = blockIdx.y;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4;
+  const int row0 = DEC ? 0 : rb * ROWS;
+  if (row0 >= m.q_len) return;
+  const int nrows = DEC ? 1 : min(ROWS, m.q_len - row0);
+  // the head of a lane's row: one head a wave for prompt portions, a head a row for decoded tokens
+  const int in_group = DEC ? blockIdx.z * 16 + l16 : blockIdx.z * kMaxWaves + w;
+  if (!DEC && in_group >= GS) return;   // (the whole wave; no barrier follows)
+  const bool head_ok = in_group < GS;
+  const int my_head = g * GS + (head_ok ? in_group : 0);
+  const int p_first = m.q_start + row0, p_last = p_first + nrows - 1;
+  const int* my_table = table + (long)m.table_row * table_stride;
+
+  bool row_ok[RT];
+  int my_pos[RT], my_lo[RT];
+  const T* q_row[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int row = DEC ? 0 : 16 * r + l16;
+    row_ok[r] = DEC ? head_ok : row < nrows;
+    my_pos[r] = p_first + (row_ok[r] ? row : 0);
+    my_lo[r] = first_seen(my_pos[r], window, chunk);
+    q_row[r] = q + (long)(m.q_off + row0 + (row_ok[r] ? row : 0)) * ldq + (long)my_head * D;
+  }
+  const float* my_bias = dist_bias ? dist_bias + (long)my_head * n_dist : nullptr;
+
+  float m_run[RT], l_run[RT];
+  f32x4 acc[RT][VB];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    m_run[r] = kNegSentinel;
+    l_run[r] = 0.f;
+#pragma unroll
+    for (int b = 0; b < VB; ++b) acc[r][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int lo_tile = first_seen(p_first, window, chunk) / kTileKeys;
+  const int hi_tile = p_last / kTileKeys;
+  const int n_tiles = hi_tile - lo_tile + 1;
+  const int per_run = (n_tiles + n_runs - 1) / n_runs;
+  const int step_end = min(n_tiles, (run + 1) * per_run);
+
+  // A tile's keys are requested while the tile before it is worked on: its addresses (page and slot of the
+  // lane's key of each half as a row of K, and of its four keys as columns of V^T) and the key vectors.
+  struct Ahead {
+    long v_at[2];
+    bool v_ok[2][4];
+    typename Atom<T>::vec_t kv[2][KCH];
+  };
+  auto request = [&](int step, Ahead& t) LS_INLINED {
+    const int key0 = (lo_tile + step) * kTileKeys;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int key = key0 + 16 * half + l16;
+      const int page = key <= p_last ? my_table[key / page_size] : -1;
+      const bool k_ok = page >= 0;
+      const long k_at = ((long)(k_ok ? page : 0) * G + g) * page_size + (k_ok ? key % page_size : 0);
+      const int key4 = key0 + 16 * half + 4 * quad;
+      const int page4 = key4 <= p_last ? my_table[key4 / page_size] : -1;
+      t.v_at[half] = ((long)(page4 >= 0 ? page4 : 0) * G + g) * DV * page_size + (page4 >= 0 ? key4 % page_size : 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.v_ok[half][i] = page4 >= 0 && key4 + i <= p_last;
+      const T* k_row = k_pages + k_at * D;
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) {
+        const bool in = c * KC + VEC * quad + VEC <= D;
+        t.kv[half][c] = load_or_zero<T>(k_row + (in ? c * KC + VEC * quad : 0), k_ok && in);
+      }
+    }
+  };
+
+  // The queries do not change from tile to tile: they stay in registers where that takes at most 64 of them.
+  constexpr bool kKeepQ = RT * KCH * (int)(sizeof(typename Atom<T>::vec_t) / 4) <= 64;
+  typename Atom<T>::vec_t qv[kKeepQ ? RT : 1][kKeepQ ? KCH : 1];
+  if constexpr (kKeepQ) {
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) {
+        const bool in = c * KC + VEC * quad + VEC <= D;
+        qv[r][c] = load_or_zero<T>(q_row[r] + (in ? c * KC + VEC * quad : 0), row_ok[r] && in);
+      }
+  }
+
+  Ahead now;
+  if (run * per_run < step_end) request(run * per_run, now);
+  for (int step = run * per_run; step < step_end; ++step) {
+    const int key0 = (lo_tile + step) * kTileKeys;
+    long v_at[2];
+    bool v_ok[2][4];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      v_at[half] = now.v_at[half];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v_ok[half][i] = now.v_ok[half][i];
+    }
+    // -- 1. transposed scores ----------------------------------------------------------------------
+    f32x4 s[RT][2];
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        s[r][half] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) {
+          if constexpr (kKeepQ) {
+            Atom<T>::mma(s[r][half], now.kv[half][c], qv[r][c]);
+          } else {
+            const bool in = c * KC + VEC * quad + VEC <= D;
+            Atom<T>::mma(s[r][half], now.kv[half][c],
+                         load_or_zero<T>(q_row[r] + (in ? c * KC + VEC * quad : 0), row_ok[r] && in));
+          }
+        }
+      }
+    if (step + 1 < step_end) request(step + 1, now);  // (the products above have taken this tile's keys)
+    // -- 2. scale, bias, mask, online softmax ------------------------------------------------------------
+    float shrink[RT];
+    bool moved = false;
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      bool see[2][4];
+      float top = kNegSentinel;
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = key0 + 16 * half + 4 * quad + i;
+          see[half][i] = row_ok[r] && key <= my_pos[r] && key >= my_lo[r];
+          float v = s[r][half][i] * scale;
+          if (my_bias) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
+          s[r][half][i] = v;
+          top = fmaxf(top, see[half][i] ? v : kNegSentinel);
+        }
+      top = quad16_max(top);
+      const float m_new = fmaxf(m_run[r], top);
+      shrink[r] = softmax_exp<T>(m_run[r] - m_new);
+      float sum = 0.f;
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          s[r][half][i] = see[half][i] ? softmax_exp<T>(s[r][half][i] - m_new) : 0.f;
+          sum = sum + s[r][half][i];
+        }
+      sum = quad16_sum(sum);
+      l_run[r] = l_run[r] * shrink[r] + sum;
+      m_run[r] = m_new;
+      moved = moved || shrink[r] != 1.0f;
+    }
+    // -- 3. values: column 16 b + l16 of V^T, keys 4 quad .. 4 quad + 3 of each half ----------------
+    bool held = true;
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) held = held && v_ok[half][i];
+    const bool all_held = __all(held) != 0 && DV % 16 == 0;
+    if (__all(!moved) == 0) {
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int b = 0; b < VB; ++b)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[r][b][i] = acc[r][b][i] * shrink[r];
+    }
+    typename Atom<T>::vec_t pb[RT][sizeof(T) == 2 ? 1 : 2];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pb[r][0][i] = (bf16_t)s[r][0][i];
+          pb[r][0][4 + i] = (bf16_t)s[r][1][i];
+        }
+      } else {
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pb[r][half][i] = s[r][half][i];
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < VB; ++b) {
+      const bool col_ok = 16 * b + l16 < DV;
+      const long column = (long)(col_ok ? 16 * b + l16 : 0) * page_size;
+      if constexpr (sizeof(T) == 2) {
+        const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[0] + column);
+        const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[1] + column);
+        bf16x8 a;
+        if (all_held) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            a[i] = v0[i];
+            a[4 + i] = v1[i];
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            a[i] = (v_ok[0][i] && col_ok) ? v0[i] : (bf16_t)0.f;
+            a[4 + i] = (v_ok[1][i] && col_ok) ? v1[i] : (bf16_t)0.f;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < RT; ++r) Atom<T>::mma(acc[r][b], a, pb[r][0]);
+      } else {
+        f32x4 a[2];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const f32x4 v = *reinterpret_cast<const f32x4*>(v_pages + v_at[half] + column);
+          if (all_held) {
+            a[half] = v;
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[half][i] = (v_ok[half][i] && col_ok) ? v[i] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+#pragma unroll
+          for (int half = 0; half < 2; ++half) Atom<T>::mma(acc[r][b], a[half], pb[r][half]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    if (!row_ok[r]) continue;
+    const int row = DEC ? 0 : 16 * r + l16;
+    if (n_runs > 1) {
+      // [item][row][head][DV + 2]: the unnormalised output, then max and sum
+      float* dst = part + (((long)blockIdx.x * part_rows + row) * H + my_head) * (DV + 2);
+#pragma unroll
+      for (int b = 0; b < VB; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (16 * b + 4 * quad + i < DV) dst[16 * b + 4 * quad + i] = acc[r][b][i];
+      if (quad == 0) {
+        dst[DV] = m_run[r];
+        dst[DV + 1] = l_run[r];
+      }
+      continue;
+    }
+    // the sink joins the sum as one more score; the row's weights then add up to less than one
+    float top = m_run[r], total = l_run[r], keep = 1.0f;
+    if (sink) {
+      const float sv = sink[my_head];
+      top = fmaxf(m_run[r], sv);
+      keep = softmax_exp<T>(m_run[r] - top);
+      total = l_run[r] * keep + softmax_exp<T>(sv - top);
+    }
+    const float inv = keep / total;
+    T* dst = out + (long)(m.q_off + row0 + row) * ldo + (long)my_head * DV;
+    const float* g_row = gate ? gate + (long)(m.q_off + row0 + row) * ldg + (long)my_head * DV : nullptr;
+#pragma unroll
+    for (int b = 0; b < VB; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = 16 * b + 4 * quad + i;
+        if (c < DV) {
+          float v = acc[r][b][i] * inv;
+          if (g_row) v = v * sigmoid_f(g_row[c]);
+          dst[c] = from_f32<T>(v);
+        }
+      }
+  }
+}
+
+// Fold the runs of row blocks: a fold item (first work item, runs, first packed row, rows) names the work items
+// first .. first + runs - 1 of one row block, whose partial results are folded in ascending order for each of its
+// rows; the sink joins the sum and the gate multiplies the result.  One workgroup a (fold item, head, row).
+template <typename T>
+__global__ __launch_bounds__(64) void sink_combine_kernel(const float* __restrict__ part, int part_rows, int H,
+                                                          const int* __restrict__ folds, const float* __restrict__ sink,
+                                                          const float* __restrict__ gate, long ldg, T* __restrict__ out,
+                                                          long ldo) {
+  const int first = folds[4 * blockIdx.x], n_runs = folds[4 * blockIdx.x + 1];
+  const int row0 = folds[4 * blockIdx.x + 2], rows = folds[4 * blockIdx.x + 3];
+  const int h = blockIdx.y;
+  const long stride = (long)part_rows * H * (DV + 2);  // from a run to the next
+  for (int r = blockIdx.z; r < rows; r += gridDim.z) {
+    const float* mine = part + (((long)first * part_rows + r) * H + h) * (DV + 2);
+    float top = sink ? sink[h] : kNegSentinel;
+    for (int k = 0; k < n_runs; ++k) top = fmaxf(top, mine[k * stride + DV]);
+    float total = 0.f;
+    for (int k = 0; k < n_runs; ++k) total = total + mine[k * stride + DV + 1] * softmax_exp<T>(mine[k * stride + DV] - top);
+    if (sink) total = total + softmax_exp<T>(sink[h] - top);
+    const float inv = 1.0f / total;
+    for (int c = threadIdx.x; c < DV; c += 64) {
+      float sum = 0.f;
+      for (int k = 0; k < n_runs; ++k) sum = sum + mine[k * stride + c] * softmax_exp<T>(mine[k * stride + DV] - top);
+      float v = sum * inv;
+      if (gate) v = v * sigmoid_f(gate[(long)(row0 + r) * ldg + (long)h * DV + c]);
+      out[(long)(row0 + r) * ldo + h * DV + c] = from_f32<T>(v);
+    }
+  }
+}
+
+}  // namespace ls
+
+LS_DEFINE_ERROR_API
+
+using namespace ls;
+
+extern "C" int ls_sink_dim() { return D; }
+extern "C" int ls_sink_vdim() { return DV; }
+extern "C" int ls_sink_max_row_tiles() { return 4; }
+
+// q [T][ldq] (H heads of D); key pages [pages][G][page_size][D], value pages [pages][G][DV][page_size]; table
+// [slots][table_stride]; seqs: the step's requests; items: n_items work items of four ints (request of the step,
+// block of 16 row_tiles of its rows, run, runs); row_tiles 1, 2 or 4, or 0 for a step of single decoded tokens.
+// sink [H] float or null; dist_bias [H][n_dist] float or null; gate: float [T][ldg] (H heads of DV) or null;
+// out [T][ldo].  Work items with runs > 1 leave their results in part (n_items * part_rows * H * (DV + 2) floats;
+// part_rows 16 row_tiles, or 1 for decoded tokens) and the n_folds fold items of four ints (first work item, runs,
+// first packed row, rows) say which to fold into which rows of out in a second launch.
+extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages,
+                                 int page_size, const int* table, int table_stride, const void* seqs,
+                                 const int* items, int n_items, int row_tiles, int H, int G, float scale, int window,
+                                 int chunk, const float* sink, const float* dist_bias, int n_dist, const float* gate,
+                                 long ldg, void* out, long ldo, const int* folds, int n_folds, float* part,
+                                 int part_rows, void* stream) {
+  LS_REQUIRE(row_tiles == 0 || row_tiles == 1 || row_tiles == 2 || row_tiles == 4, "sink_attention: %d row tiles", row_tiles);
+  LS_REQUIRE(part_rows == (row_tiles ? 16 * row_tiles : 1), "sink_attention: partial results of %d rows", part_rows);
+  LS_REQUIRE(n_folds >= 0 && (n_folds == 0 || (part && folds)), "sink_attention: %d fold items need partial results", n_folds);
+  LS_REQUIRE(n_items > 0 && q && k_pages && v_pages && table && seqs && items && out, "sink_attention: null operand");
+  LS_REQUIRE(H > 0 && G > 0 && H % G == 0, "sink_attention: %d query heads over %d key/value heads", H, G);
+  LS_REQUIRE(ldq >= (long)H * D && ldo >= (long)H * DV && (!gate || ldg >= (long)H * DV), "sink_attention: rows are too short");
+  LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && table_stride > 0, "sink_attention: page size %d", page_size);
+  LS_REQUIRE(window >= 0 && chunk >= 0 && (!dist_bias || n_dist > 0), "sink_attention: window %d, chunk %d, %d distances",
+             window, chunk, n_dist);
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(v_pages) % 16 == 0,
+             "sink_attention: operands must be 16-byte aligned");
+  LS_REQUIRE(dtype == kF32 || dtype == kBF16, "sink_attention: unknown dtype %d", dtype);
+  LS_REQUIRE(ldq % (dtype == kF32 ? 4 : 8) == 0, "sink_attention: query rows must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int GS = H / G;
+#define LS_SINK_LAUNCH(T_, RT_, DEC_)                                                                                  \
+  hipLaunchKernelGGL((sink_attention_kernel<T_, RT_, DEC_>),                                                           \
+                     dim3(n_items, G, DEC_ ? (GS + 15) / 16 : (GS + kMaxWaves - 1) / kMaxWaves),                       \
+                     dim3(DEC_ ? 64 : 64 * (GS < kMaxWaves ? GS : kMaxWaves)), 0, s, (const T_*)q, ldq,                \
+                     (const T_*)k_pages, (const T_*)v_pages, page_size, table, table_stride, (const SeqMeta*)seqs,     \
+                     items, H, G, scale, window, chunk, sink, dist_bias, n_dist, gate, ldg, (T_*)out, ldo, part,       \
+                     part_rows)
+#define LS_SINK_BY_ROWS(T_)                       \
+  switch (row_tiles) {                            \
+    case 0: LS_SINK_LAUNCH(T_, 1, true); break;   \
+    case 1: LS_SINK_LAUNCH(T_, 1, false); break;  \
+    case 2: LS_SINK_LAUNCH(T_, 2, false); break;  \
+    default: LS_SINK_LAUNCH(T_, 4, false); break; \
+  }
+  if (dtype == kF32) {
+    LS_SINK_BY_ROWS(float)
+    if (n_folds > 0)
+      hipLaunchKernelGGL(sink_combine_kernel<float>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows, H,
+                         folds, sink, gate, ldg, (float*)out, ldo);
+  } else {
+    LS_SINK_BY_ROWS(bf16_t)
+    if (n_folds > 0)
+      hipLaunchKernelGGL(sink_combine_kernel<bf16_t>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows, H,
+                         folds, sink, gate, ldg, (bf16_t*)out, ldo);
+  }
+#undef LS_SINK_BY_ROWS
+#undef LS_SINK_LAUNCH
+  return check_launch("sink_attention");
+}

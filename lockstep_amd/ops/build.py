@@ -11,6 +11,11 @@ Two kinds of library exist:
                     recurrence with per-row gates and what surrounds it;
 ``talking<shape>``  attention whose heads' scores are mixed before the softmax,
                     for one shape (query heads, kv heads, key and value size).
+``sink<D>x<DV>``    grouped-query attention with a sink in the softmax, windows or
+                    chunks of keys, a bias by distance and an output gate, for one
+                    key size and one value size;
+``experts``         routing of tokens to a few of many small feed-forward experts
+                    and the grouped products of those experts.
 
 A library's file name carries a hash of its sources and flags, so a stale
 build is never loaded.  Libraries are written next to the package
@@ -45,6 +50,8 @@ CORE_SOURCES = ("core.hip", "gemm.hip", "sample.hip")
 ATTENTION_SOURCES = ("attention.hip",)
 MIXERS_SOURCES = ("mixers.hip",)
 TALKING_SOURCES = ("talking_attention.hip",)
+SINK_SOURCES = ("sink_attention.hip",)
+EXPERTS_SOURCES = ("experts.hip",)
 
 
 class BuildError(RuntimeError):
@@ -217,6 +224,17 @@ def build_talking(heads: int, kv_heads: int, dim: int, vdim: int, force: bool = 
                   f"-DLS_TA_VDIM={vdim}"), force)
 
 
+def build_sink(dim: int, vdim: int, force: bool = False) -> Path:
+    """The sink attention library of one key size and one value size."""
+    if dim % 8 or not 8 <= dim <= 256 or vdim % 4 or not 4 <= vdim <= 256:
+        raise BuildError(f"key size {dim} / value size {vdim} are not supported: multiples of 8 / of 4, up to 256")
+    return build(f"sink{dim}x{vdim}", SINK_SOURCES, (f"-DLS_SA_DIM={dim}", f"-DLS_SA_VDIM={vdim}"), force)
+
+
+def build_experts(force: bool = False) -> Path:
+    return build("experts", EXPERTS_SOURCES, (), force)
+
+
 MUTANT_DEFINE = "-DLS_MUTANTS"
 
 
@@ -234,14 +252,18 @@ DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
 MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the controls
 #: (query heads, kv heads, key size, value size) of the talking-heads attention the tests and measurements use
 DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128))
+#: (key size, value size) of the sink attention the tests and measurements use
+DEFAULT_SINK_SHAPES = ((16, 16), (32, 16), (24, 24), (40, 40), (32, 32), (128, 128))
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True,
-              talking_shapes=DEFAULT_TALKING_SHAPES) -> list[Path]:
+              talking_shapes=DEFAULT_TALKING_SHAPES, sink_shapes=DEFAULT_SINK_SHAPES) -> list[Path]:
     """Compile the core library, the mixers library, the attention library of each head size and the
-    talking-heads attention library of each shape, a few at a time; with ``mutants`` also the control
+    talking-heads attention library of each shape, the sink attention
+    library of each key and value size and the experts library, a few at a time; with ``mutants`` also the control
     libraries of the tests."""
-    jobs = [lambda: build_core(force), lambda: build_mixers(force)]
+    jobs = [lambda: build_core(force), lambda: build_mixers(force), lambda: build_experts(force)]
+    jobs += [lambda shape=shape: build_sink(*shape, force) for shape in sink_shapes]
     jobs += [lambda d=d: build_attention(d, force) for d in head_dims]
     jobs += [lambda shape=shape: build_talking(*shape, force) for shape in talking_shapes]
     if mutants:

@@ -83,6 +83,10 @@ class Kernels:
         self.mixers_path = None
         self._talking: dict[tuple, ctypes.CDLL] = {}
         self.talking_paths: dict[tuple, str] = {}
+        self._sink: dict[tuple, ctypes.CDLL] = {}
+        self.sink_paths: dict[tuple, str] = {}
+        self._experts = None
+        self.experts_path = None
         self._argmax_scratch: dict = {}
         self._sample_scratch: dict = {}
         self._sample_scratch_kept: list = []
@@ -918,6 +922,193 @@ class Kernels:
             c_int(DTYPE_CODE[out.dtype]), _ptr(x), c_long(x.stride(0)), c_int(x.shape[0]), c_int(heads), c_int(vdim),
             _ptr(weight), _ptr(gate), c_long(ldg), c_float(eps), _ptr(out), c_long(out.stride(0)), _stream()))
 
+
+    # -- attention with a sink, and what comes before it --------------------------------------
+    def sink_lib(self, dim: int, vdim: int):
+        """The sink attention library of one key size and one value size."""
+        shape = (dim, vdim)
+        lib = self._sink.get(shape)
+        if lib is None:
+            path = _build.build_sink(*shape)
+            lib = ctypes.CDLL(str(path))
+            lib.ls_last_error.restype = ctypes.c_char_p
+            if (lib.ls_sink_dim(), lib.ls_sink_vdim()) != shape:
+                raise KernelError(f"{path} was built for another shape")
+            self._sink[shape] = lib
+            self.sink_paths[shape] = str(path)
+        return lib
+
+    def qkv_post(self, raw: torch.Tensor, n_tokens: int, heads: int, kv_heads: int, dim: int, vdim: int, bias, q_norm,
+                 k_norm, eps: float, cos, sin, rot: int, neighbours: bool, max_pos: int, tok_seq, tok_pos, seqs, table,
+                 q_out: torch.Tensor, k_pages, v_pages, page_size: int, keys_are_values: bool = False) -> None:
+        """Post pass of the fused projection ``raw`` (float32, ``q | k | v | ...``; no ``v`` with
+        ``keys_are_values``, where the biased, unnormalised keys are stored as the values): biases, a
+        root-mean-square norm over the whole of q and of k with the weights ``q_norm`` / ``k_norm``, rotation of
+        the first ``rot`` dimensions of each head in pairs ``(i, i + rot/2)`` or of ``neighbours``, queries to
+        ``q_out``, keys and values to their pages."""
+        _rows_ok(raw, "qkv_post raw"); _rows_ok(q_out, "qkv_post q_out")
+        width = heads * dim + kv_heads * dim + (0 if keys_are_values else kv_heads * vdim)
+        if not (raw.dtype == torch.float32 and raw.shape[0] >= n_tokens and raw.shape[1] >= width):
+            raise KernelError(f"qkv_post raw must be float32 [>= {n_tokens}, >= {width}]")
+        if not (q_out.dtype in DTYPE_CODE and q_out.shape[0] >= n_tokens and q_out.shape[1] == heads * dim):
+            raise KernelError("qkv_post q_out has the wrong shape or dtype")
+        if keys_are_values and dim != vdim:
+            raise KernelError(f"keys of {dim} elements cannot be values of {vdim}")
+        if bias is not None:
+            self._f32_vector(bias, width, "qkv_post bias")
+        if (q_norm is None) != (k_norm is None):
+            raise KernelError("qkv_post normalises both q and k or neither")
+        if q_norm is not None:
+            self._f32_vector(q_norm, heads * dim, "qkv_post q_norm"); self._f32_vector(k_norm, kv_heads * dim, "qkv_post k_norm")
+        positions = self._rotation_tables(cos, sin, rot, max_pos)
+        self._paged_ok(k_pages, v_pages, table, q_out.dtype, kv_heads, page_size, dim, vdim)
+        if not (max_pos // page_size < table.shape[1]):
+            raise KernelError(f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
+        for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+            if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n_tokens):
+                raise KernelError(f"{name} must be int32 with at least {n_tokens} entries")
+        if n_tokens == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_qkv_post, (
+            c_int(DTYPE_CODE[q_out.dtype]), _ptr(raw), c_long(raw.stride(0)), c_int(n_tokens), c_int(heads),
+            c_int(kv_heads), c_int(dim), c_int(vdim), c_int(int(keys_are_values)), _ptr(bias), _ptr(q_norm), _ptr(k_norm),
+            c_float(eps), _ptr(cos), _ptr(sin), c_int(rot), c_int(int(neighbours)), c_int(positions), c_int(max_pos),
+            _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table), c_int(table.shape[1]), _ptr(q_out),
+            c_long(q_out.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size), _stream()))
+
+    def sink_attention(self, q: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, k_pages, v_pages,
+                       page_size: int, table, seqs, items: torch.Tensor, n_items: int, row_tiles: int, scale: float,
+                       window: int, chunk: int, sink, dist_bias, gate, out: torch.Tensor,
+                       folds: torch.Tensor | None = None, n_folds: int = 0, part: torch.Tensor | None = None) -> None:
+        """Attention of the step's queries ``q [T, heads*dim]`` over the paged cache with a sink in the softmax.
+        ``items``: ``n_items`` work items of four ints (request of the step, block of ``16 * row_tiles`` of its
+        rows, run, runs); ``row_tiles`` 1, 2 or 4, or 0 for a step of single decoded tokens.  ``window`` /
+        ``chunk``: 0 for none.  ``sink [heads]`` float32 or None; ``dist_bias [heads, distances]`` float32 or
+        None (its last column serves every larger distance); ``gate``: float32 rows of ``heads*vdim`` logits
+        whose sigmoid multiplies the output, or None.  Row blocks whose keys are dealt to several work items
+        have a fold item in ``folds`` (first work item, runs, first packed row, rows) and their results wait in
+        ``part`` (float32) until a second launch has folded them."""
+        lib = self.sink_lib(dim, vdim)
+        _rows_ok(q, "sink_attention q"); _rows_ok(out, "sink_attention out")
+        if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype and q.shape[1] == heads * dim
+                and out.shape[1] == heads * vdim and out.shape[0] == q.shape[0]):
+            raise KernelError("sink_attention q / out have the wrong shape or dtype")
+        self._paged_ok(k_pages, v_pages, table, q.dtype, kv_heads, page_size, dim, vdim)
+        if not (items.is_cuda and items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 4 * n_items):
+            raise KernelError("sink_attention work items must hold four int32 each")
+        if row_tiles not in (0, 1, 2, 4):
+            raise KernelError(f"sink_attention takes 0, 1, 2 or 4 row tiles, got {row_tiles}")
+        part_rows = 16 * row_tiles if row_tiles else 1
+        if n_folds:
+            if not (folds is not None and folds.is_cuda and folds.dtype == torch.int32 and folds.is_contiguous()
+                    and folds.numel() >= 4 * n_folds and part is not None and part.is_cuda
+                    and part.dtype == torch.float32 and part.is_contiguous()
+                    and part.numel() >= n_items * part_rows * heads * (vdim + 2)):
+                raise KernelError("sink_attention folds: four int32 each, and room for every work item's partial result")
+        if sink is not None:
+            self._f32_vector(sink, heads, "sink_attention sink")
+        n_dist = 0
+        if dist_bias is not None:
+            if not (dist_bias.is_cuda and dist_bias.dtype == torch.float32 and dist_bias.is_contiguous()
+                    and dist_bias.dim() == 2 and dist_bias.shape[0] == heads and dist_bias.shape[1] > 0):
+                raise KernelError(f"sink_attention dist_bias must be float32 [{heads}, distances]")
+            n_dist = dist_bias.shape[1]
+        ldg = 0
+        if gate is not None:
+            _rows_ok(gate, "sink_attention gate")
+            if not (gate.dtype == torch.float32 and gate.shape[0] >= q.shape[0] and gate.shape[1] == heads * vdim):
+                raise KernelError(f"sink_attention gate must be float32 [>= {q.shape[0]}, {heads * vdim}]")
+            ldg = gate.stride(0)
+        if not (window >= 0 and chunk >= 0):
+            raise KernelError(f"sink_attention window {window} / chunk {chunk}")
+        if n_items == 0:
+            return
+        self._launch(lib, lib.ls_sink_attention, (
+            c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
+            _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items), c_int(row_tiles), c_int(heads),
+            c_int(kv_heads), c_float(scale), c_int(window), c_int(chunk), _ptr(sink), _ptr(dist_bias), c_int(n_dist),
+            _ptr(gate), c_long(ldg), _ptr(out), c_long(out.stride(0)), _ptr(folds), c_int(n_folds), _ptr(part),
+            c_int(part_rows), _stream()))
+
+    # -- many small experts --------------------------------------------------------------------
+    def experts_lib(self):
+        """The library of csrc/experts.hip, built and loaded when a part first asks for it."""
+        if self._experts is None:
+            self.experts_path = _build.build_experts()
+            lib = ctypes.CDLL(str(self.experts_path))
+            lib.ls_last_error.restype = ctypes.c_char_p
+            self._experts = lib
+        return self._experts
+
+    def experts_max_top(self) -> int:
+        return self._memo(("experts_max_top",), lambda: int(self.experts_lib().ls_experts_max_top()))
+
+    def experts_tile_capacity(self, n_tokens: int, experts: int, top: int, rows_a_tile: int) -> int:
+        """Tiles of ``rows_a_tile`` rows that the (token, choice) pairs of a step can need at most."""
+        pairs = n_tokens * top
+        return pairs // rows_a_tile + min(pairs, experts)
+
+    @staticmethod
+    def _i32(t, n: int, name: str) -> None:
+        if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n):
+            raise KernelError(f"{name} must be int32 with at least {n} elements on the GPU")
+
+    def experts_route(self, logits: torch.Tensor, bias, top: int, rows_a_tile: int, expert: torch.Tensor,
+                      weight: torch.Tensor, order: torch.Tensor, tiles: torch.Tensor, counts: torch.Tensor) -> None:
+        """From router ``logits [T, E]`` (float32) and ``bias [E]``: every token's ``top`` experts (largest logit
+        first, the lower index wins a tie) into ``expert [T, top]``, the softmax over the chosen logits into
+        ``weight [T, top]``; the pairs ``token * top + choice`` sorted by expert into ``order``, and every
+        expert's pairs cut into ``tiles [capacity, 4]`` (expert or -1, first place in ``order``, rows, 0)."""
+        _rows_ok(logits, "experts_route logits")
+        t, e = logits.shape
+        if not (logits.dtype == torch.float32 and 0 < top <= min(e, self.experts_max_top())):
+            raise KernelError(f"experts_route: float32 logits and 1 <= top <= {min(e, self.experts_max_top())}, got {top}")
+        if bias is not None:
+            self._f32_vector(bias, e, "experts_route bias")
+        cap = self.experts_tile_capacity(t, e, top, rows_a_tile)
+        self._i32(expert, t * top, "experts_route expert"); self._i32(order, t * top, "experts_route order")
+        self._i32(tiles, 4 * cap, "experts_route tiles"); self._i32(counts, e, "experts_route counts")
+        if not (weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() >= t * top):
+            raise KernelError("experts_route weight must be float32 [T, top]")
+        if t == 0:
+            return
+        lib = self.experts_lib()
+        self._launch(lib, lib.ls_experts_route, (
+            _ptr(logits), c_long(logits.stride(0)), _ptr(bias), c_int(t), c_int(e), c_int(top), c_int(rows_a_tile),
+            _ptr(expert), _ptr(weight), _ptr(order), _ptr(tiles), c_int(cap), _ptr(counts), _stream()))
+
+    def experts_apply(self, x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, top: int,
+                      rows_a_tile: int, order: torch.Tensor, tiles: torch.Tensor, weight: torch.Tensor, limit: float,
+                      alpha: float, act: torch.Tensor, partials: torch.Tensor) -> None:
+        """``partials[k][t] = weight[t, k] * down_e(act(gate_e x[t], up_e x[t]))`` for every token's ``k``-th
+        expert ``e``, with the clamped gated unit of ``glu_clamped`` as activation.  ``w_gate``, ``w_up``
+        ``[E, F, K]``, ``w_down [E, N, F]`` in the compute dtype; ``act``: scratch ``[T * top, F]`` of the
+        compute dtype; ``partials [top, T, N]`` float32; the routing as ``experts_route`` left it."""
+        _rows_ok(x, "experts_apply x"); _rows_ok(act, "experts_apply act")
+        t, k = x.shape
+        if not (w_gate.dim() == 3 and w_gate.shape == w_up.shape and w_gate.shape[2] == k and w_down.dim() == 3
+                and w_down.shape[0] == w_gate.shape[0] and w_down.shape[2] == w_gate.shape[1]
+                and w_gate.is_contiguous() and w_up.is_contiguous() and w_down.is_contiguous()
+                and w_gate.dtype == x.dtype == w_up.dtype == w_down.dtype == act.dtype and x.dtype in DTYPE_CODE):
+            raise KernelError("experts_apply weights must be [E, F, K], [E, F, K], [E, N, F] of the compute dtype")
+        e, f, n = w_gate.shape[0], w_gate.shape[1], w_down.shape[1]
+        cap = self.experts_tile_capacity(t, e, top, rows_a_tile)
+        if not (act.shape[0] >= t * top and act.shape[1] == f):
+            raise KernelError(f"experts_apply act must be [>= {t * top}, {f}]")
+        if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
+                and tuple(partials.shape) == (top, t, n)):
+            raise KernelError(f"experts_apply partials must be float32 [{top}, {t}, {n}]")
+        self._i32(order, t * top, "experts_apply order"); self._i32(tiles, 4 * cap, "experts_apply tiles")
+        if not (weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() >= t * top):
+            raise KernelError("experts_apply weight must be float32 [T, top]")
+        if t == 0:
+            return
+        lib = self.experts_lib()
+        self._launch(lib, lib.ls_experts_apply, (
+            c_int(DTYPE_CODE[x.dtype]), _ptr(x), c_long(x.stride(0)), _ptr(w_gate), _ptr(w_up), _ptr(w_down), c_int(t),
+            c_int(e), c_int(top), c_int(k), c_int(f), c_int(n), c_int(rows_a_tile), _ptr(order), _ptr(tiles), c_int(cap),
+            _ptr(weight), c_float(limit), c_float(alpha), _ptr(act), c_long(act.stride(0)), _ptr(partials), _stream()))
 
 ATTENTION_ITEM_INTS = 32
 COMBINE_ITEM_INTS = 8

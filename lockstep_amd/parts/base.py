@@ -49,7 +49,9 @@ class WeightSpec:
     32-bit arithmetic and are kept in float32; ``int`` tensors are integer
     tables kept as int32.  ``init`` steers the random-weights mode: ``normal``
     is N(0, std), ``norm`` is 1 + N(0, norm_std), ``zeros`` is 0, ``identity`` is I + N(0, std) (a
-    square matrix), ``unit`` is uniform in (0, 1).
+    square matrix), ``unit`` is uniform in (0, 1).  A dimension of -1 in ``shape`` is one that the
+    checkpoint decides (a table whose number of rows no configuration key gives); random weights
+    take ``free`` there.
     """
 
     name: str
@@ -57,19 +59,23 @@ class WeightSpec:
     kind: str = "matrix"
     init: str = "normal"
     optional: bool = False
+    free: int = 0
 
 
 @dataclass(frozen=True)
 class PagedKVSpec:
     """Keys and values of every token, or of the last ``window`` tokens; with ``keep_first`` the
     first that many tokens stay as well when the window has passed them.  ``value_dim``: the size
-    of a value where it differs from the size of a key (``head_dim``)."""
+    of a value where it differs from the size of a key (``head_dim``).  ``chunk``: queries read the
+    keys of their own run of that many positions (counted from 0) only, so everything before the
+    current run can go."""
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
     keep_first: int = 0
+    chunk: Optional[int] = None
 
     @property
     def v_dim(self) -> int:

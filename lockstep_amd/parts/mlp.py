@@ -18,7 +18,8 @@ from .base import FeedForward, PendingAdd, WeightSpec, deferred_rows, register_p
 class GatedMLP(FeedForward):
     """Parameters: ``hidden_size``, ``intermediate_size``, ``activation`` (``silu``, ``gelu``,
     ``gelu_tanh``, ``relu``), ``bias`` (optional, default False: ``gate_proj.bias``, ``up_proj.bias``
-    and ``down_proj.bias``).
+    and ``down_proj.bias``), and optionally the tensor names below the prefix, ``gate_name``,
+    ``up_name``, ``down_name`` (default ``gate_proj.weight`` and so on; biases then ``<name>.b``).
 
     SiLU without biases is the fast path (the activation is the product's epilogue).  Anything else
     stores the gate/up product in float32 and applies biases and activation in a pass of its own,
@@ -41,28 +42,36 @@ class GatedMLP(FeedForward):
         self.w_gate_up = self.w_down = self.b_gate_up = self.b_down = None
 
     @classmethod
+    def names(cls, spec: PartSpec, prefix: str):
+        """(weight, bias) tensor names of gate, up and down."""
+        out = []
+        for key, default in (("gate_name", "gate_proj"), ("up_name", "up_proj"), ("down_name", "down_proj")):
+            given = spec.params.get(key)
+            out.append((f"{prefix}.{given}", f"{prefix}.{given}.b") if given else
+                       (f"{prefix}.{default}.weight", f"{prefix}.{default}.bias"))
+        return out
+
+    @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
         h, i = int(spec["hidden_size"]), int(spec["intermediate_size"])
-        out = [WeightSpec(f"{prefix}.gate_proj.weight", (i, h)),
-               WeightSpec(f"{prefix}.up_proj.weight", (i, h)),
-               WeightSpec(f"{prefix}.down_proj.weight", (h, i))]
+        (gate, gate_b), (up, up_b), (down, down_b) = cls.names(spec, prefix)
+        out = [WeightSpec(gate, (i, h)), WeightSpec(up, (i, h)), WeightSpec(down, (h, i))]
         if spec.params.get("bias", False):
-            out += [WeightSpec(f"{prefix}.gate_proj.bias", (i,), kind="vector"),
-                    WeightSpec(f"{prefix}.up_proj.bias", (i,), kind="vector"),
-                    WeightSpec(f"{prefix}.down_proj.bias", (h,), kind="vector")]
+            out += [WeightSpec(gate_b, (i,), kind="vector"), WeightSpec(up_b, (i,), kind="vector"),
+                    WeightSpec(down_b, (h,), kind="vector")]
         return out
 
     def load(self, weights, rt) -> None:
-        gate = weights.get(f"{self.prefix}.gate_proj.weight")
-        up = weights.get(f"{self.prefix}.up_proj.weight")
+        (gate_name, gate_b), (up_name, up_b), (down_name, down_b) = self.names(self.spec, self.prefix)
+        gate = weights.get(gate_name)
+        up = weights.get(up_name)
         if gate.dtype != up.dtype:
             gate, up = gate.to(torch.float32), up.to(torch.float32)
         self.w_gate_up = rt.matrix(interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0))
-        self.w_down = rt.matrix(weights.get(f"{self.prefix}.down_proj.weight"))
+        self.w_down = rt.matrix(weights.get(down_name))
         if self.bias:
-            self.b_gate_up = rt.vector(torch.cat([weights.get(f"{self.prefix}.gate_proj.bias").to(torch.float32),
-                                                  weights.get(f"{self.prefix}.up_proj.bias").to(torch.float32)]))
-            self.b_down = rt.vector(weights.get(f"{self.prefix}.down_proj.bias"))
+            self.b_gate_up = rt.vector(torch.cat([weights.get(gate_b).to(torch.float32), weights.get(up_b).to(torch.float32)]))
+            self.b_down = rt.vector(weights.get(down_b))
 
     def forward(self, ctx, x, out, accumulate: bool, norm=None, defer: bool = False):
         """``norm``: when given, ``x`` is the float32 residual stream and ``norm``

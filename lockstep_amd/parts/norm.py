@@ -10,7 +10,8 @@ from .base import Norm, WeightSpec, register_part
 
 @register_part("rmsnorm")
 class RMSNorm(Norm):
-    """Parameters: ``size``, ``eps``; ``name`` overrides the tensor name."""
+    """Parameters: ``size``, ``eps``; ``name`` overrides the tensor name.  With ``optional`` the
+    weight may be absent (a layer whose second half is missing never runs the norm)."""
 
     graph_safe = True
     repeatable = True
@@ -27,10 +28,14 @@ class RMSNorm(Norm):
 
     @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
-        return [WeightSpec(cls.tensor_name(spec, prefix), (int(spec["size"]),), kind="vector", init="norm")]
+        return [WeightSpec(cls.tensor_name(spec, prefix), (int(spec["size"]),), kind="vector", init="norm",
+                           optional=bool(spec.params.get("optional")))]
 
     def load(self, weights, rt) -> None:
-        self.weight = rt.vector(weights.get(self.tensor_name(self.spec, self.prefix)))
+        name = self.tensor_name(self.spec, self.prefix)
+        if self.spec.params.get("optional") and name not in weights:
+            return
+        self.weight = rt.vector(weights.get(name))
 
     def forward(self, ctx, x, out, rows=None, pending=None) -> None:
         """``pending`` (a ``PendingAdd``): added to ``x`` first, in the same launch."""

@@ -1,5 +1,5 @@
-"""Rotary position encoding with half rotation: the pair of dimension ``i`` is
-``i + rotary_dim/2``.  Tables are built in float64 on the host and kept in
+"""Rotary position encoding.  ``rope_half``: the pair of dimension ``i`` is
+``i + rotary_dim/2``; ``rope_scaled`` adds a choice of the pairing and frequencies stretched by wavelength.  Tables are built in float64 on the host and kept in
 float32, ``inv_freq[i] = theta^(-2i/rotary_dim)``, ``angle = position *
 inv_freq`` (reference engine/model/qwen3.py:117-129).  The mixer applies them
 inside its fused kernel."""
@@ -63,6 +63,66 @@ class RotaryHalf(PositionEncoding):
         self._store[0] = cos.to(rt.device).contiguous()
         self._store[1] = sin.to(rt.device).contiguous()
         bump_device_epoch()
+
+
+@register_part("rope_scaled")
+class RotaryScaled(RotaryHalf):
+    """Rotary encoding with a choice of which dimensions form a pair and with frequencies that are
+    stretched by wavelength.  Parameters: ``rotary_dim`` (even), ``theta``, ``pairing`` (``"half"``:
+    dimension ``i`` with ``i + rotary_dim/2``; ``"neighbours"``: ``2i`` with ``2i + 1``) and ``scaling``
+    (None, or ``factor``, ``low``, ``high``, ``original``): with the wavelength ``l = 2 pi / f`` of a
+    pair's frequency ``f = theta^(-2i/rotary_dim)``, ``f`` stays where ``l < original/high``, becomes
+    ``f / factor`` where ``l > original/low``, and in between is ``(1 - s) f / factor + s f`` with
+    ``s = (original/l - low) / (high - low)``.
+
+    Kernels that know ``neighbours`` rotate such pairs in place; for those that pair ``i`` with
+    ``i + rotary_dim/2`` only, ``dim_order`` states the reordering of a head that brings the pairs there."""
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        super().__init__(spec, prefix)
+        self.pairing = str(spec.params.get("pairing", "half"))
+        if self.pairing not in ("half", "neighbours"):
+            raise ValueError(f"pairing {self.pairing!r} is not one of half, neighbours")
+        scaling = spec.params.get("scaling")
+        self.scaling = None
+        if scaling:
+            self.scaling = tuple(float(scaling[key]) for key in ("factor", "low", "high", "original"))
+            factor, low, high, original = self.scaling
+            if not (factor > 0 and original > 0 and high > low >= 0):
+                raise ValueError(f"frequency scaling needs factor > 0, original > 0 and high > low >= 0, got {scaling}")
+
+    @property
+    def neighbours(self) -> bool:
+        return self.pairing == "neighbours"
+
+    def share_key(self):
+        return (self.rotary_dim, self.theta, self.scaling)      # (the pairing does not enter the tables)
+
+    def frequencies(self) -> torch.Tensor:
+        import math
+
+        half = self.rotary_dim // 2
+        exponent = torch.arange(0, half, dtype=torch.float64) * 2.0 / self.rotary_dim
+        freq = 1.0 / (self.theta ** exponent)
+        if self.scaling is None:
+            return freq
+        factor, low, high, original = self.scaling
+        wavelength = 2.0 * math.pi / freq
+        blend = (original / wavelength - low) / (high - low)
+        mixed = (1.0 - blend) * freq / factor + blend * freq
+        return torch.where(wavelength * high < original, freq, torch.where(wavelength * low > original, freq / factor, mixed))
+
+    def tables(self, positions: torch.Tensor):
+        angles = positions.to(torch.float64)[:, None] * self.frequencies()[None, :]
+        return angles.cos().to(torch.float32), angles.sin().to(torch.float32)
+
+    def bind(self, rt) -> None:
+        self._store = _TABLES.setdefault((self.rotary_dim, self.theta, self.scaling, str(rt.device)), [None, None])
+
+    def dim_order(self, head_dim: int):
+        if not self.neighbours:
+            return None
+        return list(range(0, self.rotary_dim, 2)) + list(range(1, self.rotary_dim, 2)) + list(range(self.rotary_dim, head_dim))
 
 
 @register_part("no_position")

@@ -9,6 +9,7 @@ are N(0, std), norm weights are 1 + N(0, norm_std) (exactly 1 when norm_std is
 
 from __future__ import annotations
 
+import dataclasses
 import hashlib
 import json
 from pathlib import Path
@@ -38,6 +39,8 @@ def random_tensors(config: ModelConfig, seed: int, std: float | None = None, nor
         if w.name in tied:
             continue  # the tied tensor is not stored; it aliases its target
         gen = _generator(seed, w.name)
+        if any(n == -1 for n in w.shape):      # a size the checkpoint decides: the spec's own choice here
+            w = dataclasses.replace(w, shape=tuple(w.free if n == -1 else n for n in w.shape))
         if w.kind == "int":
             value = torch.zeros(w.shape, dtype=torch.int32)
         elif w.init == "norm":

@@ -66,7 +66,9 @@ def check_names_and_shapes(
             if not spec.optional:
                 missing.append(name)
             continue
-        if tuple(available[source]) != tuple(spec.shape):
+        found = tuple(available[source])
+        if len(found) != len(spec.shape) or any(want != have and not (want == -1 and have > 0)
+                                                for want, have in zip(spec.shape, found)):
             mismatched.append((name, tuple(spec.shape), tuple(available[source])))
     unexpected = sorted(n for n in available if n not in expected)
     if missing or unexpected or mismatched:
