@@ -35,8 +35,9 @@ context lengths of ``--contexts`` (default 4,096, 8,192 and 16,384 tokens).
     python bench.py --workload designs [--model qwen3-0.6b] [--layers N]
 
 measures the Bikovik design (talking-heads attention over a window that keeps the first tokens,
-HGRN2 and retention layers, Dynamic Tanh norms, a clamped gated feed-forward) beside the Qwen3
-decoder at the same layer sizes (width, feed-forward, heads, head size, layers, vocabulary), both
+HGRN2 and retention layers, Dynamic Tanh norms, a clamped gated feed-forward) and the Biberax
+design (chunked and biased attention with a sink and an output gate, routed experts; ``--designs``
+chooses) beside the Qwen3 decoder at the same layer sizes (width, feed-forward, heads, head size, layers, vocabulary), both
 with random weights: prefill of one prompt and decode steps at batch 1 and 8, each with its
 fraction of the roofline.
 """
@@ -91,7 +92,14 @@ class Workload:
             tensors = part_class(layer_spec.arrangement.kind).weight_specs(layer_spec)
             matrices = sum(_numel(w.shape) for w in tensors if w.kind == "matrix")
             vectors = sum(_numel(w.shape) for w in tensors if w.kind != "matrix")
-            per_layer.append((matrices, vectors, layer.mixer))
+            # a feed-forward of routed experts: a token multiplies with `top` of them, a step reads those it uses
+            ff = getattr(layer, "feed_forward", None)
+            routed = None
+            if getattr(ff, "experts", 0) and getattr(ff, "top", 0):
+                one = 3 * ff.inter * ff.hidden
+                matrices -= ff.experts * one
+                routed = (ff.experts, ff.top, one)
+            per_layer.append((matrices, vectors, layer.mixer, routed))
         self.runs = [per_layer[run.layer] for run in spec.schedule]
         self.writers = [per_layer[run.layer][2] for run in spec.schedule if run.writes_cache]
         self.head = spec.vocab_size * spec.hidden_size
@@ -101,14 +109,17 @@ class Workload:
         """Multiply-adds times two of a step of ``tokens`` new tokens at positions ``start``.. of
         one request with ``wanted`` logit rows."""
         total = 2.0 * wanted * self.head
-        for matrices, _, mixer in self.runs:
+        for matrices, _, mixer, routed in self.runs:
+            if routed is not None:
+                matrices = matrices + routed[1] * routed[2]
             total += 2.0 * tokens * matrices + (mixer.mixing_flops(tokens, start) if mixer is not None else 0.0)
         return total
 
     def decode_bytes(self, batch: int, context: float, element: int) -> float:
         """Bytes a decode step has to read: every weight it uses once, and what the mixers hold
         of the live requests."""
-        weights = sum(matrices * element + vectors * 4 for matrices, vectors, _ in self.runs)
+        weights = sum((matrices + (min(routed[0], batch * routed[1]) * routed[2] if routed else 0)) * element + vectors * 4
+                      for matrices, vectors, _, routed in self.runs)
         weights += self.head * element + self.hidden * 4                     # head and final norm
         weights += batch * self.hidden * element                             # embedding rows
         held = sum(batch * cache_bytes(mixer.cache_spec(), context, element) for mixer in self.writers
@@ -123,7 +134,8 @@ def cache_bytes(spec, context: float, element: int) -> float:
     if spec is None:
         return 0.0
     if isinstance(spec, PagedKVSpec):
-        return min(context, spec.window or context) * spec.num_kv_heads * (spec.head_dim + spec.v_dim) * element
+        seen = min(context, spec.window or context, getattr(spec, "chunk", None) or context)
+        return seen * spec.num_kv_heads * (spec.head_dim + spec.v_dim) * element
     if isinstance(spec, StateSpec):
         return _numel(spec.shape) * {"float32": 4, "int32": 4, "bfloat16": 2}[spec.dtype]
     raise TypeError(f"a cache unit described by {type(spec).__name__}: bench.py does not know its size")
@@ -132,7 +144,7 @@ def cache_bytes(spec, context: float, element: int) -> float:
 def _numel(shape) -> int:
     n = 1
     for size in shape:
-        n *= int(size)
+        n *= max(int(size), 0)         # (a size that only the checkpoint knows: a small table, counted as nothing)
     return n
 
 
@@ -352,8 +364,31 @@ def bikovik_like(qwen, layers: int, window: int = 4096, keep_first: int = 4):
                              "layers": [cycle[i % 4] for i in range(layers)]})
 
 
+def biberax_like(qwen, layers: int, chunk: int = 8192, experts: int = 32, top: int = 4):
+    """A Biberax configuration at the layer sizes of the Qwen3 configuration ``qwen``: the layers cycle through
+    chunked rotary attention with a dense feed-forward, the same with routed experts, the attention with shared
+    keys and values, a bias by distance and a learned sink with routed experts, and chunked attention with
+    routed experts again; every mixer has the heads and head size of the Qwen3 attention.  A token's routed
+    feed-forward multiplies with as many weights as the dense one: ``top`` experts of an eighth of half the
+    dense size each, and a shared expert of half the dense size."""
+    from lockstep_amd.config import config_from_dict
+
+    heads, kv, d = qwen.num_attention_heads, qwen.num_key_value_heads, qwen.head_dim
+    dense = {"kind": "dense", "ff": qwen.intermediate_size}
+    moe = {"kind": "moe", "expert": {"ff": qwen.intermediate_size // (2 * top), "limit": 7.0},
+           "router": {"experts": experts, "top": top}, "shared": {"ff": qwen.intermediate_size // 2, "limit": 7.0}}
+    rotary = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": chunk},
+              "rot": {"dims": d // 2, "base": qwen.rope_theta,
+                      "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    biased = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "bias_max": 4096, "bias_rows": 32}
+    cycle = [{"type": "attention", "mixer": rotary, "mlp": dense}, {"type": "attention", "mixer": rotary, "mlp": moe},
+             {"type": "attention_2", "mixer": biased, "mlp": moe}, {"type": "attention", "mixer": rotary, "mlp": moe}]
+    return config_from_dict({"architecture": "Biberax", "vocab": qwen.vocab_size, "width": qwen.hidden_size,
+                             "norm": {"eps": qwen.rms_norm_eps}, "layers": [cycle[i % 4] for i in range(layers)]})
+
+
 def designs_record(args) -> dict:
-    """Prefill and decode of the Bikovik design beside Qwen3 at equal layer sizes."""
+    """Prefill and decode of the other designs beside Qwen3 at equal layer sizes."""
     import gc
 
     import torch
@@ -369,7 +404,11 @@ def designs_record(args) -> dict:
     out = {"workload": "designs", "sizes": args.model, "layers": layers, "dtype": args.dtype,
            "prefill_tokens": args.prefill_len, "prompt_len": args.prompt_len, "steps": args.steps,
            "data": "synthetic: uniform random token ids, random weights", "designs": {}}
-    for name, config in (("qwen3", qwen), ("bikovik", bikovik_like(qwen, layers))):
+    makers = {"qwen3": lambda: qwen, "bikovik": lambda: bikovik_like(qwen, layers), "biberax": lambda: biberax_like(qwen, layers)}
+    for name in args.designs.split(","):
+        if name not in makers:
+            raise SystemExit(f"--designs: {name!r} is not one of {', '.join(makers)}")
+        config = makers[name]()
         print(f"[bench] drawing random weights for {name} at {args.model} sizes", file=sys.stderr, flush=True)
         tensors = random_tensors(config, seed=0, std=0.02, norm_std=0.0, dtype=torch.bfloat16)
         model = model_from_tensors(config, tensors, dtype=dtype)
@@ -536,8 +575,9 @@ def main(argv=None) -> int:
     p.add_argument("--workload", default="decode", choices=["decode", "serve", "reference-trace", "contexts", "designs"],
                    help="decode: fixed batches (the headline); serve / reference-trace: a workload through the "
                         "scheduler; contexts: prefill and decode at the context lengths of --contexts; designs: "
-                        "the Bikovik design beside Qwen3 at the layer sizes of --model")
+                        "the Bikovik and Biberax designs beside Qwen3 at the layer sizes of --model")
     p.add_argument("--contexts", default="4096,8192,16384", help="contexts: the context lengths, comma separated")
+    p.add_argument("--designs", default="qwen3,bikovik,biberax", help="designs: which of qwen3, bikovik, biberax, comma separated")
     p.add_argument("--repeats", type=int, default=5, help="timed runs; the median is reported with the spread")
     p.add_argument("--requests", type=int, default=0, help="serve: only the first N requests of the workload")
     p.add_argument("--prefill-chunk", type=int, default=None, help="serve: prompt portion (0: whole prompts)")

@@ -8,10 +8,10 @@
 //                 act(g, u) = g' sigmoid(alpha g') (u' + 1),  g' = min(g, limit),  u' = clamp(u, -limit, limit)
 //   P[k][t]     = w[t, k] * expert chosen(t)[k] (x[t])        (float; the caller adds the slices in order)
 //
-// Four launches.  (1) route: one thread a token picks the experts and their weights.  (2) group: the
-// (token, choice) pairs are put in the order of their experts (a stable counting sort by one workgroup:
-// a wave an expert counts its pairs by ballots, then places them), and every expert's pairs are cut
-// into tiles of ROWS rows; the tile list has a fixed capacity that depends on the sizes only, unused
+// (1) route: a wave a token picks the experts and their weights.  (2) group: the (token, choice) pairs
+// are put in the order of their experts (a stable counting sort: a wave an expert counts its pairs by
+// ballots, then places them; one workgroup does (1) and (2) for a step of few tokens), and every
+// expert's pairs are cut into tiles of ROWS rows; the tile list has a fixed capacity that depends on the sizes only, unused
 // tiles are marked.  (3) the gate and up products of every tile with the activation as epilogue; (4)
 // the down products, scaled and scattered to P.  Products use the 16x16 MFMA atom with the weight
 // rows as first operand (a lane ends with four consecutive output columns of one row); a row's
@@ -28,91 +28,156 @@ constexpr int kMaxTop = 16;
 __device__ __forceinline__ float sigmoid_e(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // ---------------------------------------------------------------------------
-// (1) One thread a token: expert [T][top] int, weight [T][top] float.
+// (1) A wave a token.  Lane l holds the logits of experts l, l + 64, ...; a pick is the best of every lane's
+// best (the larger value, then the lower index), found by exchanges across the wave; lane k < top keeps the
+// k-th pick.  expert [T][top] int, weight [T][top] float.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ z, long ldz,
-                                                         const float* __restrict__ bias, int n_tokens, int E, int top,
-                                                         int* expert, float* weight) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= n_tokens) return;
-  const float* row = z + (long)t * ldz;
-  // (the picks so far are kept in the outputs themselves: a thread reads back what it wrote)
-  int* picked = expert + (long)t * top;
-  float* value = weight + (long)t * top;
+constexpr int kMaxPerLane = 8;   // experts a lane holds: up to 512 experts
+
+__device__ __forceinline__ void pick_top(const float* __restrict__ row, const float* __restrict__ bias, int E, int top,
+                                         int lane, int* __restrict__ picked, float* __restrict__ share) {
+  float mine[kMaxPerLane];
+#pragma unroll
+  for (int m = 0; m < kMaxPerLane; ++m) {
+    const int e = lane + 64 * m;
+    mine[m] = e < E ? row[e] + (bias ? bias[e] : 0.f) : 0.f;
+  }
+  unsigned taken = 0;
+  int my_pick = 0;
+  float my_value = 0.f, first = 0.f;
   for (int k = 0; k < top; ++k) {
-    int best = -1;
     float best_v = 0.f;
-    for (int e = 0; e < E; ++e) {
-      bool taken = false;
-      for (int j = 0; j < k; ++j) taken = taken || picked[j] == e;
-      if (taken) continue;
-      const float v = row[e] + (bias ? bias[e] : 0.f);
-      if (best < 0 || v > best_v) {
+    int best = 0x7fffffff;
+#pragma unroll
+    for (int m = 0; m < kMaxPerLane; ++m) {
+      const int e = lane + 64 * m;
+      if (e < E && !((taken >> m) & 1u) && (best == 0x7fffffff || mine[m] > best_v)) {
+        best_v = mine[m];
         best = e;
-        best_v = v;
       }
     }
-    picked[k] = best;
-    value[k] = best_v;
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) {
+      const float other_v = __shfl_xor(best_v, step, kWave);
+      const int other = __shfl_xor(best, step, kWave);
+      const bool take = other != 0x7fffffff && (best == 0x7fffffff || other_v > best_v || (other_v == best_v && other < best));
+      best_v = take ? other_v : best_v;
+      best = take ? other : best;
+    }
+    if ((best & 63) == lane) taken |= 1u << (best >> 6);
+    if (k == 0) first = best_v;
+    if (lane == k) {
+      my_pick = best;
+      my_value = best_v;
+    }
   }
-  const float largest = value[0];
-  float sum = 0.f;
-  for (int k = 0; k < top; ++k) {
-    const float ex = expf(value[k] - largest);
-    value[k] = ex;
-    sum = sum + ex;
+  const float ex = lane < top ? expf(my_value - first) : 0.f;   // (the first pick is the largest)
+  const float sum = wave_sum(ex);
+  if (lane < top) {
+    picked[lane] = my_pick;
+    share[lane] = ex / sum;
   }
-  for (int k = 0; k < top; ++k) value[k] = value[k] / sum;
+}
+
+__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ z, long ldz,
+                                                         const float* __restrict__ bias, int n_tokens, int E, int top,
+                                                         int* __restrict__ expert, float* __restrict__ weight) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= n_tokens) return;
+  pick_top(z + (long)t * ldz, bias, E, top, threadIdx.x & 63, expert + (long)t * top, weight + (long)t * top);
 }
 
 // ---------------------------------------------------------------------------
-// (2) One workgroup of 16 waves.  order [P]: the pairs (token * top + choice) sorted by expert, stable.
-// tiles [cap][4]: expert (-1: unused), first place in order, rows, 0.
+// (2) order [P]: the pairs (token * top + choice) sorted by expert, stable.  tiles [cap][4]: expert (-1: unused),
+// first place in order, rows, 0.  A wave an expert: it counts its pairs by ballots, adds up the counts of the
+// experts before it, writes its tiles and places its pairs.  Many pairs: two launches of a wave an expert
+// (count; place).  Few: one workgroup that also picks the experts, with the picks and counts in LDS.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void route_group_kernel(const int* __restrict__ expert, int P, int E, int rows_a_tile,
-                                                           int* __restrict__ order, int* __restrict__ tiles, int cap,
-                                                           int* __restrict__ counts) {
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  // counts [E] (pairs of an expert), then their running sums; in global scratch: E has no bound here
-  for (int e = w; e < E; e += 16) {
-    int n = 0;
-    for (int p0 = 0; p0 < P; p0 += 64) {
-      const bool mine = p0 + lane < P && expert[p0 + lane] == e;
-      n += __popcll(__ballot(mine));
+__device__ __forceinline__ int count_pairs(const int* expert, int P, int e, int lane) {
+  int n = 0;
+  for (int p0 = 0; p0 < P; p0 += 64) {
+    const bool mine = p0 + lane < P && expert[p0 + lane] == e;
+    n += __popcll(__ballot(mine));
+  }
+  return n;
+}
+
+__device__ __forceinline__ void place_pairs(const int* expert, const int* counts, int P, int E, int e, int lane,
+                                            int rows_a_tile, int* __restrict__ order, int* __restrict__ tiles, int cap) {
+  int base = 0, tile = 0;
+  for (int j0 = 0; j0 < e; j0 += 64) {   // (sums of whole numbers: any order)
+    const int c = j0 + lane < e ? counts[j0 + lane] : 0;
+    int b = c, t = (c + rows_a_tile - 1) / rows_a_tile;
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) {
+      b += __shfl_xor(b, step, kWave);
+      t += __shfl_xor(t, step, kWave);
     }
-    if (lane == 0) counts[e] = n;
+    base += b;
+    tile += t;
+  }
+  const int n = counts[e];
+  for (int i = lane; i * rows_a_tile < n; i += 64) {
+    if (tile + i < cap) {
+      tiles[4 * (tile + i)] = e;
+      tiles[4 * (tile + i) + 1] = base + i * rows_a_tile;
+      tiles[4 * (tile + i) + 2] = min(rows_a_tile, n - i * rows_a_tile);
+      tiles[4 * (tile + i) + 3] = 0;
+    }
+  }
+  if (e == E - 1) {
+    const int used = tile + (n + rows_a_tile - 1) / rows_a_tile;
+    for (int i = used + lane; i < cap; i += 64) {
+      tiles[4 * i] = -1;
+      tiles[4 * i + 1] = tiles[4 * i + 2] = tiles[4 * i + 3] = 0;
+    }
+  }
+  int at = base;
+  for (int p0 = 0; p0 < P; p0 += 64) {
+    const bool mine = p0 + lane < P && expert[p0 + lane] == e;
+    const unsigned long long votes = __ballot(mine);
+    if (mine) order[at + __popcll(votes & ((1ull << lane) - 1ull))] = p0 + lane;
+    at += __popcll(votes);
+  }
+}
+
+__global__ __launch_bounds__(64) void route_count_kernel(const int* __restrict__ expert, int P, int* __restrict__ counts) {
+  const int n = count_pairs(expert, P, blockIdx.x, threadIdx.x);
+  if (threadIdx.x == 0) counts[blockIdx.x] = n;
+}
+
+__global__ __launch_bounds__(64) void route_place_kernel(const int* __restrict__ expert, const int* __restrict__ counts,
+                                                         int P, int E, int rows_a_tile, int* __restrict__ order,
+                                                         int* __restrict__ tiles, int cap) {
+  place_pairs(expert, counts, P, E, blockIdx.x, threadIdx.x, rows_a_tile, order, tiles, cap);
+}
+
+constexpr int kSmallPairs = 2048, kSmallExperts = 512;   // what the one-workgroup kernel keeps in LDS
+
+__global__ __launch_bounds__(1024) void route_small_kernel(const float* __restrict__ z, long ldz,
+                                                           const float* __restrict__ bias, int n_tokens, int E, int top,
+                                                           int rows_a_tile, int* __restrict__ expert,
+                                                           float* __restrict__ weight, int* __restrict__ order,
+                                                           int* __restrict__ tiles, int cap) {
+  __shared__ int picks_s[kSmallPairs];
+  __shared__ float share_s[16][kMaxTop];
+  __shared__ int counts_s[kSmallExperts];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int P = n_tokens * top;
+  for (int t = w; t < n_tokens; t += 16) {
+    pick_top(z + (long)t * ldz, bias, E, top, lane, picks_s + t * top, share_s[w]);
+    if (lane < top) {
+      expert[(long)t * top + lane] = picks_s[t * top + lane];
+      weight[(long)t * top + lane] = share_s[w][lane];
+    }
   }
   __syncthreads();
   for (int e = w; e < E; e += 16) {
-    int base = 0, tile = 0;
-    for (int j = 0; j < e; ++j) {      // (every lane the same few additions)
-      base += counts[j];
-      tile += (counts[j] + rows_a_tile - 1) / rows_a_tile;
-    }
-    const int n = counts[e];
-    for (int i = lane; i * rows_a_tile < n; i += 64) {
-      if (tile + i < cap) {
-        tiles[4 * (tile + i)] = e;
-        tiles[4 * (tile + i) + 1] = base + i * rows_a_tile;
-        tiles[4 * (tile + i) + 2] = min(rows_a_tile, n - i * rows_a_tile);
-        tiles[4 * (tile + i) + 3] = 0;
-      }
-    }
-    if (e == E - 1) {
-      const int used = tile + (n + rows_a_tile - 1) / rows_a_tile;
-      for (int i = used + lane; i < cap; i += 64) {
-        tiles[4 * i] = -1;
-        tiles[4 * i + 1] = tiles[4 * i + 2] = tiles[4 * i + 3] = 0;
-      }
-    }
-    int at = base;
-    for (int p0 = 0; p0 < P; p0 += 64) {
-      const bool mine = p0 + lane < P && expert[p0 + lane] == e;
-      const unsigned long long votes = __ballot(mine);
-      if (mine) order[at + __popcll(votes & ((1ull << lane) - 1ull))] = p0 + lane;
-      at += __popcll(votes);
-    }
+    const int n = count_pairs(picks_s, P, e, lane);
+    if (lane == 0) counts_s[e] = n;
   }
+  __syncthreads();
+  for (int e = w; e < E; e += 16) place_pairs(picks_s, counts_s, P, E, e, lane, rows_a_tile, order, tiles, cap);
 }
 
 // ---------------------------------------------------------------------------
@@ -148,16 +213,25 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
 #pragma unroll
   for (int r = 0; r < RT; ++r) acc_g[r] = acc_u[r] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bool aligned = K % VEC == 0;
-  for (int k0 = 0; k0 < K; k0 += KC) {
-    const int k = k0 + VEC * quad;
-    const typename Atom<T>::vec_t a_g = load_vec<T>(g_row, 0, k, K, 0, w_ok, aligned);
-    const typename Atom<T>::vec_t a_u = load_vec<T>(u_row, 0, k, K, 0, w_ok, aligned);
+  // the operands of U chunks are requested together, then multiplied in ascending order
+  constexpr int U = RT == 1 ? 8 : 4;
+  for (int k0 = 0; k0 < K; k0 += U * KC) {
+    typename Atom<T>::vec_t a_g[U], a_u[U], b[U][RT];
 #pragma unroll
-    for (int r = 0; r < RT; ++r) {
-      const typename Atom<T>::vec_t b = load_vec<T>(x_row[r], 0, k, K, 0, x_ok[r], aligned);
-      Atom<T>::mma(acc_g[r], a_g, b);
-      Atom<T>::mma(acc_u[r], a_u, b);
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * KC + VEC * quad;
+      a_g[u] = load_vec<T>(g_row, 0, k, K, 0, w_ok, aligned);
+      a_u[u] = load_vec<T>(u_row, 0, k, K, 0, w_ok, aligned);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) b[u][r] = load_vec<T>(x_row[r], 0, k, K, 0, x_ok[r], aligned);
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < RT; ++r) {
+        Atom<T>::mma(acc_g[r], a_g[u], b[u][r]);
+        Atom<T>::mma(acc_u[r], a_u[u], b[u][r]);
+      }
   }
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
@@ -205,11 +279,20 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
 #pragma unroll
   for (int r = 0; r < RT; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bool aligned = F % VEC == 0 && ldy % VEC == 0;
-  for (int k0 = 0; k0 < F; k0 += KC) {
-    const int k = k0 + VEC * quad;
-    const typename Atom<T>::vec_t a = load_vec<T>(d_row, 0, k, F, 0, w_ok, aligned);
+  constexpr int U = RT == 1 ? 8 : 4;
+  for (int k0 = 0; k0 < F; k0 += U * KC) {
+    typename Atom<T>::vec_t a[U], b[U][RT];
 #pragma unroll
-    for (int r = 0; r < RT; ++r) Atom<T>::mma(acc[r], a, load_vec<T>(y_row[r], 0, k, F, 0, y_ok[r], aligned));
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * KC + VEC * quad;
+      a[u] = load_vec<T>(d_row, 0, k, F, 0, w_ok, aligned);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) b[u][r] = load_vec<T>(y_row[r], 0, k, F, 0, y_ok[r], aligned);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < RT; ++r) Atom<T>::mma(acc[r], a[u], b[u][r]);
   }
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
@@ -249,11 +332,18 @@ extern "C" int ls_experts_route(const float* z, long ldz, const float* bias, int
   LS_REQUIRE(rows_a_tile == 16 || rows_a_tile == 32 || rows_a_tile == 64, "experts_route: tiles of %d rows", rows_a_tile);
   LS_REQUIRE(z && expert && weight && order && tiles && counts, "experts_route: null operand");
   LS_REQUIRE(cap >= ls_experts_tile_capacity(n_tokens, E, top, rows_a_tile), "experts_route: %d tiles are too few", cap);
+  LS_REQUIRE(E <= 64 * kMaxPerLane, "experts_route: %d experts, the routing kernel takes %d", E, 64 * kMaxPerLane);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 255) / 256), dim3(256), 0, s, z, ldz, bias, n_tokens, E, top,
-                     expert, weight);
-  hipLaunchKernelGGL(route_group_kernel, dim3(1), dim3(1024), 0, s, expert, n_tokens * top, E, rows_a_tile, order, tiles,
-                     cap, counts);
+  const int P = n_tokens * top;
+  if (P <= kSmallPairs && E <= kSmallExperts) {
+    hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(1024), 0, s, z, ldz, bias, n_tokens, E, top, rows_a_tile,
+                       expert, weight, order, tiles, cap);
+  } else {
+    hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, s, z, ldz, bias, n_tokens, E, top,
+                       expert, weight);
+    hipLaunchKernelGGL(route_count_kernel, dim3(E), dim3(64), 0, s, expert, P, counts);
+    hipLaunchKernelGGL(route_place_kernel, dim3(E), dim3(64), 0, s, expert, counts, P, E, rows_a_tile, order, tiles, cap);
+  }
   return check_launch("experts_route");
 }
 

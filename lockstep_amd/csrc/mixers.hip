@@ -164,7 +164,8 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 //   q and k rotated on their first `rot` dimensions at the token's position, pairs (i, i + rot/2) or, with
 //   `neighbours`, (2i, 2i + 1), angle tables [positions][rot/2];
 //   q -> q_out [T][H*D] (T);  k -> key pages [page][G][slot][D];  v -> value pages [page][G][DV][slot].
-// One workgroup a token.  The sums of squares: thread t adds the squares of elements t, t + 256, ... in
+// A token's row is dealt to workgroups of 256 elements (each forms the row's sums of squares itself where a norm
+// is asked for).  The sums of squares: thread t adds the squares of elements t, t + 256, ... in
 // ascending order, then a butterfly over the wave and the wave sums in wave order: a function of the sizes only.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float block_sum256(float v, float* scratch) {
@@ -231,13 +232,20 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
     }
     return own;
   };
-  for (int e = threadIdx.x; e < nq; e += 256) q_out[(long)t * ldq + e] = from_f32<T>(finished(e));
-  if (page < 0) return;
-  for (int e = threadIdx.x; e < nk; e += 256) {
-    const int g = e / D, i = e % D;
-    k_pages[(((long)page * G + g) * page_size + slot) * D + i] = from_f32<T>(finished(nq + e));
+  // blockIdx.y walks the row in pieces of 256 elements of q | k | v: one element a thread
+  const int e = blockIdx.y * 256 + threadIdx.x;
+  if (e < nq) {
+    q_out[(long)t * ldq + e] = from_f32<T>(finished(e));
+    return;
   }
-  for (int c = threadIdx.x; c < nv; c += 256) {
+  if (page < 0) return;
+  if (e < nq + nk) {
+    const int g = (e - nq) / D, i = (e - nq) % D;
+    k_pages[(((long)page * G + g) * page_size + slot) * D + i] = from_f32<T>(finished(e));
+    return;
+  }
+  const int c = e - nq - nk;
+  if (c < nv) {
     const int from = keys_are_values ? nq + c : nq + nk + c;
     const float v = row[from] + (bias ? bias[from] : 0.f);
     const int g = c / DV, i = c % DV;
@@ -594,7 +602,7 @@ extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, i
   LS_REQUIRE((q_norm == nullptr) == (k_norm == nullptr) && (!q_norm || eps > 0.f), "qkv_post: bad norm");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 #define LS_QKV_POST(T_)                                                                                               \
-  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens), dim3(256), 0, s, raw, ld, H, G, D, DV, keys_are_values,     \
+  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens, (unsigned)((width + (keys_are_values ? (long)G * DV : 0) + 255) / 256)), dim3(256), 0, s, raw, ld, H, G, D, DV, keys_are_values,     \
                      bias, q_norm, k_norm, eps, cos_table, sin_table, rot, neighbours, tok_seq, tok_pos,              \
                      (const SeqMeta*)seqs, table, table_stride, (T_*)q_out, ldq, (T_*)k_pages, (T_*)v_pages, page_size)
   if (dtype == kF32)

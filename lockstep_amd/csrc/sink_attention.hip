@@ -30,6 +30,8 @@
 
 #include "common.h"
 
+#include <type_traits>
+
 #ifndef LS_SA_DIM
 #error "compile with -DLS_SA_DIM and -DLS_SA_VDIM"
 #endif
@@ -124,11 +126,15 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
   const int step_end = min(n_tiles, (run + 1) * per_run);
 
   // A tile's keys are requested while the tile before it is worked on: its addresses (page and slot of the
-  // lane's key of each half as a row of K, and of its four keys as columns of V^T) and the key vectors.
+  // lane's key of each half as a row of K, and of its four keys as columns of V^T), the key vectors and the values.
+  typedef typename std::conditional<sizeof(T) == 2, bf16x4, f32x4>::type v4_t;   // four keys of one value column
+  // (the values travel with the keys where the registers allow it: not with four row tiles of wide values)
+  constexpr bool kAheadV = RT * VB <= 16;
   struct Ahead {
     long v_at[2];
     bool v_ok[2][4];
     typename Atom<T>::vec_t kv[2][KCH];
+    v4_t vv[2][kAheadV ? VB : 1];
   };
   auto request = [&](int step, Ahead& t) LS_INLINED {
     const int key0 = (lo_tile + step) * kTileKeys;
@@ -140,7 +146,8 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
       const long k_at = ((long)(k_ok ? page : 0) * G + g) * page_size + (k_ok ? key % page_size : 0);
       const int key4 = key0 + 16 * half + 4 * quad;
       const int page4 = key4 <= p_last ? my_table[key4 / page_size] : -1;
-      t.v_at[half] = ((long)(page4 >= 0 ? page4 : 0) * G + g) * DV * page_size + (page4 >= 0 ? key4 % page_size : 0);
+      const long v_at = ((long)(page4 >= 0 ? page4 : 0) * G + g) * DV * page_size + (page4 >= 0 ? key4 % page_size : 0);
+      t.v_at[half] = v_at;
 #pragma unroll
       for (int i = 0; i < 4; ++i) t.v_ok[half][i] = page4 >= 0 && key4 + i <= p_last;
       const T* k_row = k_pages + k_at * D;
@@ -148,6 +155,13 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
       for (int c = 0; c < KCH; ++c) {
         const bool in = c * KC + VEC * quad + VEC <= D;
         t.kv[half][c] = load_or_zero<T>(k_row + (in ? c * KC + VEC * quad : 0), k_ok && in);
+      }
+      if constexpr (kAheadV) {   // (the values too: they are on their way while the scores are formed)
+#pragma unroll
+        for (int b = 0; b < VB; ++b) {
+          const long column = (long)(16 * b + l16 < DV ? 16 * b + l16 : 0) * page_size;
+          t.vv[half][b] = *reinterpret_cast<const v4_t*>(v_pages + v_at + column);
+        }
       }
     }
   };
@@ -169,13 +183,18 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
   if (run * per_run < step_end) request(run * per_run, now);
   for (int step = run * per_run; step < step_end; ++step) {
     const int key0 = (lo_tile + step) * kTileKeys;
-    long v_at[2];
     bool v_ok[2][4];
+    long v_at[2];
+    v4_t vv[2][kAheadV ? VB : 1];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       v_at[half] = now.v_at[half];
 #pragma unroll
       for (int i = 0; i < 4; ++i) v_ok[half][i] = now.v_ok[half][i];
+      if constexpr (kAheadV) {
+#pragma unroll
+        for (int b = 0; b < VB; ++b) vv[half][b] = now.vv[half][b];
+      }
     }
     // -- 1. transposed scores ----------------------------------------------------------------------
     f32x4 s[RT][2];
@@ -265,9 +284,15 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
     for (int b = 0; b < VB; ++b) {
       const bool col_ok = 16 * b + l16 < DV;
       const long column = (long)(col_ok ? 16 * b + l16 : 0) * page_size;
+      auto value4 = [&](int half) LS_INLINED {
+        if constexpr (kAheadV) {
+          return vv[half][b];
+        } else {
+          return *reinterpret_cast<const v4_t*>(v_pages + v_at[half] + column);
+        }
+      };
       if constexpr (sizeof(T) == 2) {
-        const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[0] + column);
-        const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(v_pages + v_at[1] + column);
+        const bf16x4 v0 = value4(0), v1 = value4(1);
         bf16x8 a;
         if (all_held) {
 #pragma unroll
@@ -288,7 +313,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
         f32x4 a[2];
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-          const f32x4 v = *reinterpret_cast<const f32x4*>(v_pages + v_at[half] + column);
+          const f32x4 v = value4(half);
           if (all_held) {
             a[half] = v;
           } else {
@@ -359,17 +384,37 @@ __global__ __launch_bounds__(64) void sink_combine_kernel(const float* __restric
   const int row0 = folds[4 * blockIdx.x + 2], rows = folds[4 * blockIdx.x + 3];
   const int h = blockIdx.y;
   const long stride = (long)part_rows * H * (DV + 2);  // from a run to the next
+  __shared__ float factor_s[64];
   for (int r = blockIdx.z; r < rows; r += gridDim.z) {
     const float* mine = part + (((long)first * part_rows + r) * H + h) * (DV + 2);
+    // lane k holds run k's statistics (runs <= 64): all of them are requested at once
+    const int k_mine = threadIdx.x;
+    const float m_k = k_mine < n_runs ? mine[k_mine * stride + DV] : kNegSentinel;
+    const float l_k = k_mine < n_runs ? mine[k_mine * stride + DV + 1] : 0.f;
     float top = sink ? sink[h] : kNegSentinel;
-    for (int k = 0; k < n_runs; ++k) top = fmaxf(top, mine[k * stride + DV]);
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) top = fmaxf(top, __shfl_xor(top, step, kWave));
+    float top_runs = m_k;
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) top_runs = fmaxf(top_runs, __shfl_xor(top_runs, step, kWave));
+    top = fmaxf(top, top_runs);
+    const float f_k = k_mine < n_runs ? softmax_exp<T>(m_k - top) : 0.f;
+    __syncthreads();
+    factor_s[k_mine] = f_k;
     float total = 0.f;
-    for (int k = 0; k < n_runs; ++k) total = total + mine[k * stride + DV + 1] * softmax_exp<T>(mine[k * stride + DV] - top);
+    for (int k = 0; k < n_runs; ++k) total = total + __shfl(l_k, k, kWave) * __shfl(f_k, k, kWave);   // ascending
     if (sink) total = total + softmax_exp<T>(sink[h] - top);
     const float inv = 1.0f / total;
+    __syncthreads();
     for (int c = threadIdx.x; c < DV; c += 64) {
       float sum = 0.f;
-      for (int k = 0; k < n_runs; ++k) sum = sum + mine[k * stride + c] * softmax_exp<T>(mine[k * stride + DV] - top);
+      int k = 0;
+      for (; k + 4 <= n_runs; k += 4) {
+        const float p0 = mine[k * stride + c], p1 = mine[(k + 1) * stride + c], p2 = mine[(k + 2) * stride + c],
+                    p3 = mine[(k + 3) * stride + c];
+        sum = (((sum + p0 * factor_s[k]) + p1 * factor_s[k + 1]) + p2 * factor_s[k + 2]) + p3 * factor_s[k + 3];
+      }
+      for (; k < n_runs; ++k) sum = sum + mine[k * stride + c] * factor_s[k];
       float v = sum * inv;
       if (gate) v = v * sigmoid_f(gate[(long)(row0 + r) * ldg + (long)h * DV + c]);
       out[(long)(row0 + r) * ldo + h * DV + c] = from_f32<T>(v);
