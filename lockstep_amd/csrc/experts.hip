@@ -95,9 +95,12 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ int count_pairs(const int* expert, int P, int e, int lane) {
   int n = 0;
-  for (int p0 = 0; p0 < P; p0 += 64) {
-    const bool mine = p0 + lane < P && expert[p0 + lane] == e;
-    n += __popcll(__ballot(mine));
+  for (int p0 = 0; p0 < P; p0 += 256) {   // (four loads requested together)
+    int got[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) got[u] = p0 + 64 * u + lane < P ? expert[p0 + 64 * u + lane] : -1;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) n += __popcll(__ballot(got[u] == e));
   }
   return n;
 }
@@ -133,11 +136,17 @@ __device__ __forceinline__ void place_pairs(const int* expert, const int* counts
     }
   }
   int at = base;
-  for (int p0 = 0; p0 < P; p0 += 64) {
-    const bool mine = p0 + lane < P && expert[p0 + lane] == e;
-    const unsigned long long votes = __ballot(mine);
-    if (mine) order[at + __popcll(votes & ((1ull << lane) - 1ull))] = p0 + lane;
-    at += __popcll(votes);
+  for (int p0 = 0; p0 < P; p0 += 256) {
+    int got[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) got[u] = p0 + 64 * u + lane < P ? expert[p0 + 64 * u + lane] : -1;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const bool mine = got[u] == e;
+      const unsigned long long votes = __ballot(mine);
+      if (mine) order[at + __popcll(votes & ((1ull << lane) - 1ull))] = p0 + 64 * u + lane;
+      at += __popcll(votes);
+    }
   }
 }
 
@@ -152,7 +161,7 @@ __global__ __launch_bounds__(64) void route_place_kernel(const int* __restrict__
   place_pairs(expert, counts, P, E, blockIdx.x, threadIdx.x, rows_a_tile, order, tiles, cap);
 }
 
-constexpr int kSmallPairs = 2048, kSmallExperts = 512;   // what the one-workgroup kernel keeps in LDS
+constexpr int kSmallPairs = 512, kSmallExperts = 512;   // what the one-workgroup kernel keeps in LDS
 
 __global__ __launch_bounds__(1024) void route_small_kernel(const float* __restrict__ z, long ldz,
                                                            const float* __restrict__ bias, int n_tokens, int E, int top,
@@ -184,7 +193,7 @@ __global__ __launch_bounds__(1024) void route_small_kernel(const float* __restri
 // (3) act [P][ldy] (T) = act(x[token] W_gate[e]^T, x[token] W_up[e]^T) for the pairs of every tile, in the
 // order of `order`.  w_gate, w_up [E][F][K].  A workgroup: one tile, four waves with 16 columns of F each.
 // ---------------------------------------------------------------------------
-template <typename T, int RT>
+template <typename T, int RT, int KS>
 __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restrict__ x, long ldx,
                                                               const T* __restrict__ w_gate, const T* __restrict__ w_up,
                                                               int F, int K, int top, const int* __restrict__ order,
@@ -196,7 +205,9 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
   const int first = tiles[4 * blockIdx.x + 1], rows = tiles[4 * blockIdx.x + 2];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int l16 = lane & 15, quad = lane >> 4;
-  const int col0 = (blockIdx.y * 4 + w) * 16;
+  // KS 1: the four waves take 16 columns each.  KS 4 (few rows): they take a quarter of K each for the same 16
+  // columns, so that all of a wave's operands are on their way at once, and their sums are added in wave order.
+  const int col0 = KS == 1 ? (blockIdx.y * 4 + w) * 16 : blockIdx.y * 16;
   if (col0 >= F) return;
   const bool w_ok = col0 + l16 < F;
   const T* g_row = w_gate + ((long)e * F + (w_ok ? col0 + l16 : 0)) * K;
@@ -215,15 +226,17 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
   const bool aligned = K % VEC == 0;
   // the operands of U chunks are requested together, then multiplied in ascending order
   constexpr int U = RT == 1 ? 8 : 4;
-  for (int k0 = 0; k0 < K; k0 += U * KC) {
+  const int k_each = KS == 1 ? K : (K + KC * KS - 1) / (KC * KS) * KC;
+  const int k_lo = KS == 1 ? 0 : w * k_each, k_hi = KS == 1 ? K : min(K, k_lo + k_each);
+  for (int k0 = k_lo; k0 < k_hi; k0 += U * KC) {
     typename Atom<T>::vec_t a_g[U], a_u[U], b[U][RT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = k0 + u * KC + VEC * quad;
-      a_g[u] = load_vec<T>(g_row, 0, k, K, 0, w_ok, aligned);
-      a_u[u] = load_vec<T>(u_row, 0, k, K, 0, w_ok, aligned);
+      a_g[u] = load_vec<T>(g_row, 0, k, k_hi, 0, w_ok, aligned);
+      a_u[u] = load_vec<T>(u_row, 0, k, k_hi, 0, w_ok, aligned);
 #pragma unroll
-      for (int r = 0; r < RT; ++r) b[u][r] = load_vec<T>(x_row[r], 0, k, K, 0, x_ok[r], aligned);
+      for (int r = 0; r < RT; ++r) b[u][r] = load_vec<T>(x_row[r], 0, k, k_hi, 0, x_ok[r], aligned);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -232,6 +245,25 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
         Atom<T>::mma(acc_g[r], a_g[u], b[u][r]);
         Atom<T>::mma(acc_u[r], a_u[u], b[u][r]);
       }
+  }
+  if constexpr (KS > 1) {
+    __shared__ f32x4 sums_s[KS][2][RT][64];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      sums_s[w][0][r][lane] = acc_g[r];
+      sums_s[w][1][r][lane] = acc_u[r];
+    }
+    __syncthreads();
+    if (w != 0) return;
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int o = 1; o < KS; ++o)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc_g[r][i] = acc_g[r][i] + sums_s[o][0][r][lane][i];
+          acc_u[r][i] = acc_u[r][i] + sums_s[o][1][r][lane][i];
+        }
   }
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
@@ -252,7 +284,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
 // ---------------------------------------------------------------------------
 // (4) P[choice][token][:] = weight[pair] * (act[place] W_down[e]^T).  w_down [E][N][F]; P [top][n_tokens][N] float.
 // ---------------------------------------------------------------------------
-template <typename T, int RT>
+template <typename T, int RT, int KS>
 __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__ act, long ldy,
                                                            const T* __restrict__ w_down, int N, int F, int top,
                                                            int n_tokens, const int* __restrict__ order,
@@ -264,7 +296,7 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
   const int first = tiles[4 * blockIdx.x + 1], rows = tiles[4 * blockIdx.x + 2];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int l16 = lane & 15, quad = lane >> 4;
-  const int col0 = (blockIdx.y * 4 + w) * 16;
+  const int col0 = KS == 1 ? (blockIdx.y * 4 + w) * 16 : blockIdx.y * 16;
   if (col0 >= N) return;
   const bool w_ok = col0 + l16 < N;
   const T* d_row = w_down + ((long)e * N + (w_ok ? col0 + l16 : 0)) * F;
@@ -280,19 +312,34 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
   for (int r = 0; r < RT; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bool aligned = F % VEC == 0 && ldy % VEC == 0;
   constexpr int U = RT == 1 ? 8 : 4;
-  for (int k0 = 0; k0 < F; k0 += U * KC) {
+  const int k_each = KS == 1 ? F : (F + KC * KS - 1) / (KC * KS) * KC;
+  const int k_lo = KS == 1 ? 0 : w * k_each, k_hi = KS == 1 ? F : min(F, k_lo + k_each);
+  for (int k0 = k_lo; k0 < k_hi; k0 += U * KC) {
     typename Atom<T>::vec_t a[U], b[U][RT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = k0 + u * KC + VEC * quad;
-      a[u] = load_vec<T>(d_row, 0, k, F, 0, w_ok, aligned);
+      a[u] = load_vec<T>(d_row, 0, k, k_hi, 0, w_ok, aligned);
 #pragma unroll
-      for (int r = 0; r < RT; ++r) b[u][r] = load_vec<T>(y_row[r], 0, k, F, 0, y_ok[r], aligned);
+      for (int r = 0; r < RT; ++r) b[u][r] = load_vec<T>(y_row[r], 0, k, k_hi, 0, y_ok[r], aligned);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int r = 0; r < RT; ++r) Atom<T>::mma(acc[r], a[u], b[u][r]);
+  }
+  if constexpr (KS > 1) {
+    __shared__ f32x4 sums_s[KS][RT][64];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) sums_s[w][r][lane] = acc[r];
+    __syncthreads();
+    if (w != 0) return;
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int o = 1; o < KS; ++o)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[r][i] = acc[r][i] + sums_s[o][r][lane][i];
   }
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
@@ -364,19 +411,21 @@ extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* 
                  reinterpret_cast<uintptr_t>(w_down) % 16 == 0 && (K % vec != 0 || ldx % vec == 0),
              "experts_apply: operands must be 16-byte aligned");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const dim3 grid_up(cap, (F + 63) / 64), grid_down(cap, (N + 63) / 64);
-#define LS_EXPERTS(T_, RT_)                                                                                           \
+  // tiles of 16 rows (few tokens an expert): a workgroup takes 16 columns and cuts K over its waves
+  const int cols = rows_a_tile == 16 ? 16 : 64;
+  const dim3 grid_up(cap, (F + cols - 1) / cols), grid_down(cap, (N + cols - 1) / cols);
+#define LS_EXPERTS(T_, RT_, KS_)                                                                                      \
   do {                                                                                                                \
-    hipLaunchKernelGGL((experts_gate_up_kernel<T_, RT_>), grid_up, dim3(256), 0, s, (const T_*)x, ldx,                \
+    hipLaunchKernelGGL((experts_gate_up_kernel<T_, RT_, KS_>), grid_up, dim3(256), 0, s, (const T_*)x, ldx,           \
                        (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, (T_*)act, ldy);     \
-    hipLaunchKernelGGL((experts_down_kernel<T_, RT_>), grid_down, dim3(256), 0, s, (const T_*)act, ldy,               \
+    hipLaunchKernelGGL((experts_down_kernel<T_, RT_, KS_>), grid_down, dim3(256), 0, s, (const T_*)act, ldy,          \
                        (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
   } while (0)
 #define LS_EXPERTS_BY_ROWS(T_)                 \
   switch (rows_a_tile) {                       \
-    case 16: LS_EXPERTS(T_, 1); break;         \
-    case 32: LS_EXPERTS(T_, 2); break;         \
-    default: LS_EXPERTS(T_, 4); break;         \
+    case 16: LS_EXPERTS(T_, 1, 4); break;      \
+    case 32: LS_EXPERTS(T_, 2, 1); break;      \
+    default: LS_EXPERTS(T_, 4, 1); break;      \
   }
   if (dtype == kF32) {
     LS_EXPERTS_BY_ROWS(float)

@@ -232,24 +232,22 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
     }
     return own;
   };
-  // blockIdx.y walks the row in pieces of 256 elements of q | k | v: one element a thread
-  const int e = blockIdx.y * 256 + threadIdx.x;
-  if (e < nq) {
-    q_out[(long)t * ldq + e] = from_f32<T>(finished(e));
-    return;
-  }
-  if (page < 0) return;
-  if (e < nq + nk) {
-    const int g = (e - nq) / D, i = (e - nq) % D;
-    k_pages[(((long)page * G + g) * page_size + slot) * D + i] = from_f32<T>(finished(e));
-    return;
-  }
-  const int c = e - nq - nk;
-  if (c < nv) {
-    const int from = keys_are_values ? nq + c : nq + nk + c;
-    const float v = row[from] + (bias ? bias[from] : 0.f);
-    const int g = c / DV, i = c % DV;
-    v_pages[(((long)page * G + g) * DV + i) * page_size + slot] = from_f32<T>(v);
+  // the workgroups of a token (gridDim.y of them) deal its elements of q | k | v among themselves, 256 at a time
+  for (int e = blockIdx.y * 256 + threadIdx.x; e < nq + nk + nv; e += gridDim.y * 256) {
+    if (e < nq) {
+      q_out[(long)t * ldq + e] = from_f32<T>(finished(e));
+    } else if (page < 0) {
+      break;
+    } else if (e < nq + nk) {
+      const int g = (e - nq) / D, i = (e - nq) % D;
+      k_pages[(((long)page * G + g) * page_size + slot) * D + i] = from_f32<T>(finished(e));
+    } else {
+      const int c = e - nq - nk;
+      const int from = keys_are_values ? nq + c : nq + nk + c;
+      const float v = row[from] + (bias ? bias[from] : 0.f);
+      const int g = c / DV, i = c % DV;
+      v_pages[(((long)page * G + g) * DV + i) * page_size + slot] = from_f32<T>(v);
+    }
   }
 }
 
@@ -601,8 +599,12 @@ extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, i
   LS_REQUIRE(max_pos / page_size < table_stride, "qkv_post: position %d is beyond the block table", max_pos);
   LS_REQUIRE((q_norm == nullptr) == (k_norm == nullptr) && (!q_norm || eps > 0.f), "qkv_post: bad norm");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // Without a norm every element stands alone: a thread an element.  With one, every workgroup of a token forms the
+  // row's sums itself, so a step of many tokens gives each token one workgroup, and a few tokens are spread out.
+  const unsigned all = (unsigned)((width + (keys_are_values ? (long)G * DV : 0) + 255) / 256);
+  const unsigned pieces = !q_norm ? all : (n_tokens <= 64 ? all : 1u);
 #define LS_QKV_POST(T_)                                                                                               \
-  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens, (unsigned)((width + (keys_are_values ? (long)G * DV : 0) + 255) / 256)), dim3(256), 0, s, raw, ld, H, G, D, DV, keys_are_values,     \
+  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens, pieces), dim3(256), 0, s, raw, ld, H, G, D, DV, keys_are_values,     \
                      bias, q_norm, k_norm, eps, cos_table, sin_table, rot, neighbours, tok_seq, tok_pos,              \
                      (const SeqMeta*)seqs, table, table_stride, (T_*)q_out, ldq, (T_*)k_pages, (T_*)v_pages, page_size)
   if (dtype == kF32)

@@ -119,6 +119,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
     for (int b = 0; b < VB; ++b) acc[r][b] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
+  const int lo_last = first_seen(p_last, window, chunk);   // (no row of the block begins to see later than this)
   const int lo_tile = first_seen(p_first, window, chunk) / kTileKeys;
   const int hi_tile = p_last / kTileKeys;
   const int n_tiles = hi_tile - lo_tile + 1;
@@ -216,39 +217,48 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
       }
     if (step + 1 < step_end) request(step + 1, now);  // (the products above have taken this tile's keys)
     // -- 2. scale, bias, mask, online softmax ------------------------------------------------------------
+    // A tile that every row of the block sees whole (most tiles of a long prompt) needs no mask: the same for the
+    // whole wave, so the choice costs a scalar branch.
     float shrink[RT];
     bool moved = false;
+    auto softmax_tile = [&](auto whole) LS_INLINED {
+      constexpr bool kWhole = decltype(whole)::value;
 #pragma unroll
-    for (int r = 0; r < RT; ++r) {
-      bool see[2][4];
-      float top = kNegSentinel;
+      for (int r = 0; r < RT; ++r) {
+        bool see[2][4];
+        float top = kNegSentinel;
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
+        for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = key0 + 16 * half + 4 * quad + i;
-          see[half][i] = row_ok[r] && key <= my_pos[r] && key >= my_lo[r];
-          float v = s[r][half][i] * scale;
-          if (my_bias) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
-          s[r][half][i] = v;
-          top = fmaxf(top, see[half][i] ? v : kNegSentinel);
-        }
-      top = quad16_max(top);
-      const float m_new = fmaxf(m_run[r], top);
-      shrink[r] = softmax_exp<T>(m_run[r] - m_new);
-      float sum = 0.f;
+          for (int i = 0; i < 4; ++i) {
+            const int key = key0 + 16 * half + 4 * quad + i;
+            see[half][i] = kWhole || (row_ok[r] && key <= my_pos[r] && key >= my_lo[r]);
+            float v = s[r][half][i] * scale;
+            if (my_bias) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
+            s[r][half][i] = v;
+            top = fmaxf(top, see[half][i] ? v : kNegSentinel);
+          }
+        top = quad16_max(top);
+        const float m_new = fmaxf(m_run[r], top);
+        shrink[r] = softmax_exp<T>(m_run[r] - m_new);
+        float sum = 0.f;
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
+        for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          s[r][half][i] = see[half][i] ? softmax_exp<T>(s[r][half][i] - m_new) : 0.f;
-          sum = sum + s[r][half][i];
-        }
-      sum = quad16_sum(sum);
-      l_run[r] = l_run[r] * shrink[r] + sum;
-      m_run[r] = m_new;
-      moved = moved || shrink[r] != 1.0f;
-    }
+          for (int i = 0; i < 4; ++i) {
+            s[r][half][i] = see[half][i] ? softmax_exp<T>(s[r][half][i] - m_new) : 0.f;
+            sum = sum + s[r][half][i];
+          }
+        sum = quad16_sum(sum);
+        l_run[r] = l_run[r] * shrink[r] + sum;
+        m_run[r] = m_new;
+        moved = moved || shrink[r] != 1.0f;
+      }
+    };
+    if (key0 + kTileKeys - 1 <= p_first && key0 >= lo_last)
+      softmax_tile(std::true_type{});
+    else
+      softmax_tile(std::false_type{});
     // -- 3. values: column 16 b + l16 of V^T, keys 4 quad .. 4 quad + 3 of each half ----------------
     bool held = true;
 #pragma unroll
