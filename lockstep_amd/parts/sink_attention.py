@@ -154,8 +154,9 @@ class SinkAttention(Mixer):
             self.sink = rt.vector(torch.zeros(self.nq, dtype=torch.float32))
         if self.distance_bias is not None:
             table = weights.get(f"{self.prefix}.rel").to(torch.float32)            # [B, H]
-            if table.dim() != 2 or table.shape[0] < 2 or table.shape[0] % 2:
-                raise ValueError(f"{self.prefix}.rel must have an even number of rows (at least 2), got {tuple(table.shape)}")
+            if table.dim() != 2 or table.shape[0] < 2 or float(self.distance_bias["farthest"]) <= table.shape[0] // 2:
+                raise ValueError(f"{self.prefix}.rel must have at least two rows and its farthest distance must lie beyond "
+                                 f"the first half of them, got {tuple(table.shape)} and {self.distance_bias['farthest']}")
             rows = distance_buckets(table.shape[0], float(self.distance_bias["farthest"]))
             self.by_distance = rt.vector(table[torch.tensor(rows)].T.contiguous())   # [H, distances]
         rt.kernels.mixers_lib()

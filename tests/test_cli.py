@@ -67,3 +67,20 @@ def test_init_writes_a_bikovik_folder_from_its_preset(tmp_path):
     names = SafetensorsFile(tmp_path / "k" / "model.safetensors").keys()
     for name in ("embed", "head", "final.norm.alpha", "l0.mix.lower", "l1.mix.talk", "l3.mix.vmix", "l2.mix.g", "l2.mlp.down"):
         assert name in names, name
+
+
+def test_init_writes_a_biberax_folder_from_its_preset(tmp_path):
+    from lockstep_amd.config import BiberaxConfig, config_from_dir
+    from lockstep_amd.weights import SafetensorsFile
+
+    done = run("init", "--preset", "biberax-tiny", "--out", str(tmp_path / "k"), "--seed", "2")
+    assert done.returncode == 0, done.stderr
+    config = config_from_dir(tmp_path / "k")
+    assert isinstance(config, BiberaxConfig) and config.width == 128 and len(config.layers) == 4
+    handle = SafetensorsFile(tmp_path / "k" / "model.safetensors")
+    names = handle.keys()
+    for name in ("embed", "head", "final.norm", "l0.mix.g", "l0.mlp.gate", "l1.mix.rel", "l1.mix.sink", "l1.mix.q.norm",
+                 "l1.mlp.e7.down", "l1.mlp.router.b", "l2.mlp.shared.up", "l3.mix.o.b"):
+        assert name in names, name
+    assert "l1.mix.v" not in names and "l3.mlp.gate" not in names
+    assert tuple(handle.shape("l1.mix.rel")) == (16, 4)
