@@ -163,7 +163,8 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 //   vector: x / sqrt(mean(x^2) + eps)), times a weight an element (q_norm [H*D], k_norm [G*D]; null: no norm);
 //   q and k rotated on their first `rot` dimensions at the token's position, pairs (i, i + rot/2) or, with
 //   `neighbours`, (2i, 2i + 1), angle tables [positions][rot/2];
-//   q -> q_out [T][H*D] (T);  k -> key pages [page][G][slot][D];  v -> value pages [page][G][DV][slot].
+//   q -> q_out [T][H*Dp] (T);  k -> key pages [page][G][slot][Dp], Dp >= D with zeros beyond D (a kernel that loads
+//   16 bytes at a time wants heads of a multiple of that);  v -> value pages [page][G][DV][slot].
 // A token's row is dealt to workgroups of 256 elements (each forms the row's sums of squares itself where a norm
 // is asked for).  The sums of squares: thread t adds the squares of elements t, t + 256, ... in
 // ascending order, then a butterfly over the wave and the wave sums in wave order: a function of the sizes only.
@@ -179,7 +180,7 @@ __device__ __forceinline__ float block_sum256(float v, float* scratch) {
 
 template <typename T>
 __global__ __launch_bounds__(256) void qkv_post_kernel(
-    const float* __restrict__ raw, long ld, int H, int G, int D, int DV, int keys_are_values,
+    const float* __restrict__ raw, long ld, int H, int G, int D, int Dp, int DV, int keys_are_values,
     const float* __restrict__ bias, const float* __restrict__ q_norm, const float* __restrict__ k_norm, float eps,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot, int neighbours,
     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, const SeqMeta* __restrict__ seqs,
@@ -232,17 +233,20 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
     }
     return own;
   };
-  // the workgroups of a token (gridDim.y of them) deal its elements of q | k | v among themselves, 256 at a time
-  for (int e = blockIdx.y * 256 + threadIdx.x; e < nq + nk + nv; e += gridDim.y * 256) {
-    if (e < nq) {
-      q_out[(long)t * ldq + e] = from_f32<T>(finished(e));
+  // the workgroups of a token (gridDim.y of them) deal its elements of q | k | v among themselves, 256 at a time;
+  // queries and keys are written with Dp >= D elements a head, zeros beyond D
+  const int oq = H * Dp, ok = G * Dp;
+  for (int e = blockIdx.y * 256 + threadIdx.x; e < oq + ok + nv; e += gridDim.y * 256) {
+    if (e < oq) {
+      const int head = e / Dp, i = e % Dp;
+      q_out[(long)t * ldq + e] = from_f32<T>(i < D ? finished(head * D + i) : 0.f);
     } else if (page < 0) {
       break;
-    } else if (e < nq + nk) {
-      const int g = (e - nq) / D, i = (e - nq) % D;
-      k_pages[(((long)page * G + g) * page_size + slot) * D + i] = from_f32<T>(finished(e));
+    } else if (e < oq + ok) {
+      const int g = (e - oq) / Dp, i = (e - oq) % Dp;
+      k_pages[(((long)page * G + g) * page_size + slot) * Dp + i] = from_f32<T>(i < D ? finished(nq + g * D + i) : 0.f);
     } else {
-      const int c = e - nq - nk;
+      const int c = e - oq - ok;
       const int from = keys_are_values ? nq + c : nq + nk + c;
       const float v = row[from] + (bias ? bias[from] : 0.f);
       const int g = c / DV, i = c % DV;
@@ -581,16 +585,16 @@ extern "C" int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, i
   return check_launch("talk_qkv");
 }
 
-extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int DV,
+extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int Dp, int DV,
                            int keys_are_values, const float* bias, const float* q_norm, const float* k_norm, float eps,
                            const float* cos_table, const float* sin_table, int rot, int neighbours,
                            int table_positions, int max_pos, const int* tok_seq, const int* tok_pos, const void* seqs,
                            const int* table, int table_stride, void* q_out, long ldq, void* k_pages, void* v_pages,
                            int page_size, void* stream) {
-  LS_REQUIRE(n_tokens > 0 && H > 0 && G > 0 && D > 0 && DV > 0 && H % G == 0, "qkv_post: bad head sizes");
+  LS_REQUIRE(n_tokens > 0 && H > 0 && G > 0 && D > 0 && Dp >= D && DV > 0 && H % G == 0, "qkv_post: bad head sizes");
   LS_REQUIRE(!keys_are_values || DV == D, "qkv_post: keys of %d elements cannot be values of %d", D, DV);
   const long width = (long)H * D + (long)G * D + (keys_are_values ? 0 : (long)G * DV);
-  LS_REQUIRE(ld >= width && ldq >= (long)H * D && raw && q_out && k_pages && v_pages && table && seqs && tok_seq &&
+  LS_REQUIRE(ld >= width && ldq >= (long)H * Dp && raw && q_out && k_pages && v_pages && table && seqs && tok_seq &&
                  tok_pos && page_size > 0 && table_stride > 0,
              "qkv_post: bad operands");
   LS_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "qkv_post: %d rotated dimensions of %d", rot, D);
@@ -601,10 +605,10 @@ extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, i
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   // Without a norm every element stands alone: a thread an element.  With one, every workgroup of a token forms the
   // row's sums itself, so a step of many tokens gives each token one workgroup, and a few tokens are spread out.
-  const unsigned all = (unsigned)((width + (keys_are_values ? (long)G * DV : 0) + 255) / 256);
+  const unsigned all = (unsigned)(((long)(H + G) * Dp + (long)G * DV + 255) / 256);
   const unsigned pieces = !q_norm ? all : (n_tokens <= 64 ? all : 1u);
 #define LS_QKV_POST(T_)                                                                                               \
-  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens, pieces), dim3(256), 0, s, raw, ld, H, G, D, DV, keys_are_values,     \
+  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens, pieces), dim3(256), 0, s, raw, ld, H, G, D, Dp, DV, keys_are_values, \
                      bias, q_norm, k_norm, eps, cos_table, sin_table, rot, neighbours, tok_seq, tok_pos,              \
                      (const SeqMeta*)seqs, table, table_stride, (T_*)q_out, ldq, (T_*)k_pages, (T_*)v_pages, page_size)
   if (dtype == kF32)

@@ -32,8 +32,9 @@ int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, int H, int G
 
 // Post pass of an attention projection raw = q | k | v (| more): biases, a root-mean-square norm over the whole of q
 // and of k (weights q_norm [H*D], k_norm [G*D], or null), rotation in pairs (i, i + rot/2) or of neighbours, keys
-// that are also the values (keys_are_values: no v in raw, the biased unnormalised k is stored as v).
-int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int DV, int keys_are_values,
+// that are also the values (keys_are_values: no v in raw, the biased unnormalised k is stored as v).  Queries and
+// keys are written with Dp >= D elements a head, zeros beyond D.
+int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int Dp, int DV, int keys_are_values,
                 const float* bias, const float* q_norm, const float* k_norm, float eps, const float* cos_table,
                 const float* sin_table, int rot, int neighbours, int table_positions, int max_pos, const int* tok_seq,
                 const int* tok_pos, const void* seqs, const int* table, int table_stride, void* q_out, long ldq,

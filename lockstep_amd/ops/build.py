@@ -226,8 +226,8 @@ def build_talking(heads: int, kv_heads: int, dim: int, vdim: int, force: bool = 
 
 def build_sink(dim: int, vdim: int, force: bool = False) -> Path:
     """The sink attention library of one key size and one value size."""
-    if dim % 8 or not 8 <= dim <= 256 or vdim % 4 or not 4 <= vdim <= 256:
-        raise BuildError(f"key size {dim} / value size {vdim} are not supported: multiples of 8 / of 4, up to 256")
+    if dim % 8 or not 8 <= dim <= 256 or not 1 <= vdim <= 256:
+        raise BuildError(f"key size {dim} / value size {vdim} are not supported: a multiple of 8 up to 256 / at most 256")
     return build(f"sink{dim}x{vdim}", SINK_SOURCES, (f"-DLS_SA_DIM={dim}", f"-DLS_SA_VDIM={vdim}"), force)
 
 

@@ -940,17 +940,20 @@ class Kernels:
 
     def qkv_post(self, raw: torch.Tensor, n_tokens: int, heads: int, kv_heads: int, dim: int, vdim: int, bias, q_norm,
                  k_norm, eps: float, cos, sin, rot: int, neighbours: bool, max_pos: int, tok_seq, tok_pos, seqs, table,
-                 q_out: torch.Tensor, k_pages, v_pages, page_size: int, keys_are_values: bool = False) -> None:
+                 q_out: torch.Tensor, k_pages, v_pages, page_size: int, keys_are_values: bool = False,
+                 key_pad: int | None = None) -> None:
         """Post pass of the fused projection ``raw`` (float32, ``q | k | v | ...``; no ``v`` with
         ``keys_are_values``, where the biased, unnormalised keys are stored as the values): biases, a
         root-mean-square norm over the whole of q and of k with the weights ``q_norm`` / ``k_norm``, rotation of
         the first ``rot`` dimensions of each head in pairs ``(i, i + rot/2)`` or of ``neighbours``, queries to
-        ``q_out``, keys and values to their pages."""
+        ``q_out``, keys and values to their pages.  ``key_pad``: the size of a head in ``q_out`` and in the key
+        pages where it exceeds ``dim`` (zeros beyond ``dim``)."""
         _rows_ok(raw, "qkv_post raw"); _rows_ok(q_out, "qkv_post q_out")
+        key_pad = dim if key_pad is None else key_pad
         width = heads * dim + kv_heads * dim + (0 if keys_are_values else kv_heads * vdim)
         if not (raw.dtype == torch.float32 and raw.shape[0] >= n_tokens and raw.shape[1] >= width):
             raise KernelError(f"qkv_post raw must be float32 [>= {n_tokens}, >= {width}]")
-        if not (q_out.dtype in DTYPE_CODE and q_out.shape[0] >= n_tokens and q_out.shape[1] == heads * dim):
+        if not (key_pad >= dim and q_out.dtype in DTYPE_CODE and q_out.shape[0] >= n_tokens and q_out.shape[1] == heads * key_pad):
             raise KernelError("qkv_post q_out has the wrong shape or dtype")
         if keys_are_values and dim != vdim:
             raise KernelError(f"keys of {dim} elements cannot be values of {vdim}")
@@ -961,7 +964,7 @@ class Kernels:
         if q_norm is not None:
             self._f32_vector(q_norm, heads * dim, "qkv_post q_norm"); self._f32_vector(k_norm, kv_heads * dim, "qkv_post k_norm")
         positions = self._rotation_tables(cos, sin, rot, max_pos)
-        self._paged_ok(k_pages, v_pages, table, q_out.dtype, kv_heads, page_size, dim, vdim)
+        self._paged_ok(k_pages, v_pages, table, q_out.dtype, kv_heads, page_size, key_pad, vdim)
         if not (max_pos // page_size < table.shape[1]):
             raise KernelError(f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
         for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
@@ -972,7 +975,7 @@ class Kernels:
         lib = self.mixers_lib()
         self._launch(lib, lib.ls_qkv_post, (
             c_int(DTYPE_CODE[q_out.dtype]), _ptr(raw), c_long(raw.stride(0)), c_int(n_tokens), c_int(heads),
-            c_int(kv_heads), c_int(dim), c_int(vdim), c_int(int(keys_are_values)), _ptr(bias), _ptr(q_norm), _ptr(k_norm),
+            c_int(kv_heads), c_int(dim), c_int(key_pad), c_int(vdim), c_int(int(keys_are_values)), _ptr(bias), _ptr(q_norm), _ptr(k_norm),
             c_float(eps), _ptr(cos), _ptr(sin), c_int(rot), c_int(int(neighbours)), c_int(positions), c_int(max_pos),
             _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table), c_int(table.shape[1]), _ptr(q_out),
             c_long(q_out.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size), _stream()))

@@ -75,6 +75,7 @@ class SinkAttention(Mixer):
         self.hidden = int(p["hidden_size"])
         self.nq, self.nkv = int(p["num_heads"]), int(p["num_kv_heads"])
         self.d, self.dv = int(p["head_dim"]), int(p["value_dim"])
+        self.dk = -(-self.d // 8) * 8       # a head of the queries and of the cached keys: the kernel loads 16 bytes at a time
         self.scale = float(p["scale"])
         self.window = int(p.get("window") or 0)
         self.chunk = int(p.get("chunk") or 0)
@@ -131,7 +132,7 @@ class SinkAttention(Mixer):
         return out
 
     def cache_spec(self):
-        return PagedKVSpec(self.nkv, self.d, self.window or None, value_dim=self.dv, chunk=self.chunk or None)
+        return PagedKVSpec(self.nkv, self.dk, self.window or None, value_dim=self.dv, chunk=self.chunk or None)
 
     def load(self, weights, rt) -> None:
         names = ["q", "k"] + ([] if self.shared_kv else ["v"]) + (["g"] if self.gate else [])
@@ -160,7 +161,7 @@ class SinkAttention(Mixer):
             rows = distance_buckets(table.shape[0], float(self.distance_bias["farthest"]))
             self.by_distance = rt.vector(table[torch.tensor(rows)].T.contiguous())   # [H, distances]
         rt.kernels.mixers_lib()
-        rt.kernels.sink_lib(self.d, self.dv)
+        rt.kernels.sink_lib(self.dk, self.dv)
         if hasattr(self.position, "bind"):
             self.position.bind(rt)
 
@@ -219,7 +220,9 @@ class SinkAttention(Mixer):
             row_tiles = 0
         else:
             longest_portion = int(ctx.q_len.max())
-            row_tiles = ROW_TILES or (1 if longest_portion <= 16 else 2 if longest_portion <= 32 or ctx.n_tokens < 1024 else 4)
+            # (two row tiles a wave measure best at key sizes of 128: 16.7 ms against 18.1 with one and 17.6 with
+            # four for a prompt of 2,048 tokens at Qwen3-0.6B sizes; four remain for measurements)
+            row_tiles = ROW_TILES or (1 if longest_portion <= 16 else 2)
             block_rows = 16 * row_tiles
             counts = -(-ctx.q_len // block_rows)
             seq = np.repeat(np.arange(ctx.n_seqs), counts)
@@ -254,11 +257,11 @@ class SinkAttention(Mixer):
             raise ValueError("a sink attention layer writes its own keys and values")
         raw = ctx.buf("sink.in_f32", (t, self.w_in.shape[0]), torch.float32)
         k.gemm(x, self.w_in, raw, STORE_F32)
-        q = ctx.buf("sink.q", (t, nq * d), rt.dtype)
+        q = ctx.buf("sink.q", (t, nq * self.dk), rt.dtype)
         k.qkv_post(raw, t, nq, nkv, d, dv, self.b_in, self.q_norm, self.k_norm, self.qk_norm or 0.0, self.position.cos,
                    self.position.sin, self.position.rotary_dim, self.neighbours, ctx.max_position, ctx.tok_seq,
                    ctx.tok_pos, ctx.seqs, group.table, q, key_pages, value_pages, group.page_size,
-                   keys_are_values=self.shared_kv)
+                   keys_are_values=self.shared_kv, key_pad=self.dk)
         key = self._block_key()
         attn = ctx.buf("sink.out", (t, nq * dv), rt.dtype)
         n_items, n_folds, row_tiles = ctx.notes[key]
@@ -266,7 +269,7 @@ class SinkAttention(Mixer):
         part_rows = 16 * row_tiles if row_tiles else 1
         part = ctx.buf("sink.part", (n_items * part_rows * nq * (dv + 2),), torch.float32) if n_folds else None
         gate = raw[:, raw.shape[1] - nq * dv:] if self.gate else None
-        k.sink_attention(q, nq, nkv, d, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
+        k.sink_attention(q, nq, nkv, self.dk, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                          work[:4 * n_items], n_items, row_tiles, self.scale, self.window, self.chunk, self.sink,
                          self.by_distance, gate, attn, work[4 * n_items:] if n_folds else None, n_folds, part)
         if self.b_o is not None:

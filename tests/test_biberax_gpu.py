@@ -341,10 +341,10 @@ def test_whole_prompt_portions_and_token_by_token_agree_with_the_plain_model(mod
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_long_prompt_in_large_row_blocks_whose_keys_are_dealt_to_runs(models, dtype):
-    """A prompt of 1,100 tokens: a step that large takes row blocks of 64 rows, the late row blocks of the
-    layers that see all keys are dealt to several work items and folded (the buffer of partial results
-    exists afterwards); decoding goes on from there, also cut into runs."""
+def test_a_long_prompt_whose_keys_are_dealt_to_runs(models, dtype):
+    """A prompt of 1,100 tokens: the late row blocks of the layers that see all keys are dealt to several
+    work items and folded (the buffer of partial results exists afterwards); decoding goes on from
+    there, also cut into runs."""
     model, oracle, raw, page, _ = models("B", dtype)
     tokens = random_tokens(1120, raw["vocab"], seed=13)
     want = oracle.forward(tokens, round_router_input=torch.bfloat16 if dtype == "bfloat16" else None)
