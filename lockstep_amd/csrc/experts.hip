@@ -355,6 +355,171 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same two products for tiles of 64 rows (many tokens an expert), both operands staged through LDS: a
+// workgroup takes 64 rows x 64 columns, its four waves 32 x 32 each.  A stage is 128 bytes of K for every row of
+// the operands (two chunks of the atom), copied from global memory into registers while the stage before it is
+// multiplied, then written to the other of two LDS buffers; rows of an LDS tile are 144 bytes apart, which
+// spreads the sixteen rows of a fragment read over all banks.  A row's contraction is still one chain over
+// ascending chunks from zero: the same bits as the kernels above give without a cut of K.  NB: weight matrices
+// that share the rows (gate and up: 2; down: 1).
+// ---------------------------------------------------------------------------
+constexpr int kStageBytes = 128, kLdsRow = kStageBytes + 16;
+
+template <typename T, int NB>
+struct TiledProduct {
+  typedef typename Atom<T>::vec_t vec_t;
+  static constexpr int VEC = Atom<T>::VEC;
+  static constexpr int kStageK = kStageBytes / (int)sizeof(T);
+  vec_t staged[1 + NB][2];
+  f32x4 acc[NB][2][2];
+
+  // a_row / b_row: where this thread's two pieces of a stage come from (null: zeros), for rows tid/8 and tid/8 + 32
+  __device__ __forceinline__ void request(const T* const (&a_row)[2], const T* const (&b_row)[NB][2], int k0, int K) {
+    const int seg = threadIdx.x & 7;
+    const int k = k0 + seg * VEC;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      staged[0][j] = (a_row[j] && k < K) ? *reinterpret_cast<const vec_t*>(a_row[j] + k) : Atom<T>::zero();
+#pragma unroll
+      for (int m = 0; m < NB; ++m)
+        staged[1 + m][j] = (b_row[m][j] && k < K) ? *reinterpret_cast<const vec_t*>(b_row[m][j] + k) : Atom<T>::zero();
+    }
+  }
+  __device__ __forceinline__ void store(char* lds) {
+    const int row = threadIdx.x >> 3, seg = threadIdx.x & 7;
+#pragma unroll
+    for (int m = 0; m < 1 + NB; ++m)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        *reinterpret_cast<vec_t*>(lds + ((m * 64) + row + 32 * j) * kLdsRow + seg * 16) = staged[m][j];
+  }
+  __device__ __forceinline__ void multiply(const char* lds) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l16 = lane & 15, quad = lane >> 4, wr = w >> 1, wc = w & 1;
+#pragma unroll
+    for (int c = 0; c < kStageBytes / 64; ++c) {
+      vec_t a[2], b[NB][2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        a[t] = *reinterpret_cast<const vec_t*>(lds + (wr * 32 + t * 16 + l16) * kLdsRow + c * 64 + quad * 16);
+#pragma unroll
+        for (int m = 0; m < NB; ++m)
+          b[m][t] = *reinterpret_cast<const vec_t*>(lds + ((1 + m) * 64 + wc * 32 + t * 16 + l16) * kLdsRow + c * 64 + quad * 16);
+      }
+#pragma unroll
+      for (int m = 0; m < NB; ++m)
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) Atom<T>::mma(acc[m][rt][ct], b[m][ct], a[rt]);
+    }
+  }
+  __device__ __forceinline__ void run(const T* const (&a_row)[2], const T* const (&b_row)[NB][2], int K, char* lds) {
+#pragma unroll
+    for (int m = 0; m < NB; ++m)
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) acc[m][rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int kBuffer = (1 + NB) * 64 * kLdsRow;
+    const int stages = (K + kStageK - 1) / kStageK;
+    request(a_row, b_row, 0, K);
+    store(lds);
+    __syncthreads();
+    for (int s = 0; s < stages; ++s) {
+      if (s + 1 < stages) request(a_row, b_row, (s + 1) * kStageK, K);
+      multiply(lds + (s & 1) * kBuffer);
+      if (s + 1 < stages) store(lds + ((s + 1) & 1) * kBuffer);
+      __syncthreads();
+    }
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void experts_gate_up_tiled_kernel(const T* __restrict__ x, long ldx,
+                                                                    const T* __restrict__ w_gate,
+                                                                    const T* __restrict__ w_up, int F, int K, int top,
+                                                                    const int* __restrict__ order,
+                                                                    const int* __restrict__ tiles, float limit, float alpha,
+                                                                    T* __restrict__ act, long ldy) {
+  __shared__ __attribute__((aligned(16))) char lds[2 * 3 * 64 * kLdsRow];
+  const int e = tiles[4 * blockIdx.x];
+  if (e < 0) return;
+  const int first = tiles[4 * blockIdx.x + 1], rows = tiles[4 * blockIdx.x + 2];
+  const int col0 = blockIdx.y * 64;
+  const T* a_row[2];
+  const T* b_row[2][2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int r = (threadIdx.x >> 3) + 32 * j;
+    a_row[j] = r < rows ? x + (long)(order[first + r] / top) * ldx : nullptr;
+    b_row[0][j] = col0 + r < F ? w_gate + ((long)e * F + col0 + r) * K : nullptr;
+    b_row[1][j] = col0 + r < F ? w_up + ((long)e * F + col0 + r) * K : nullptr;
+  }
+  TiledProduct<T, 2> product;
+  product.run(a_row, b_row, K, lds);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4, wr = w >> 1, wc = w & 1;
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int r = wr * 32 + rt * 16 + l16;
+    if (r >= rows) continue;
+    T* dst = act + (long)(first + r) * ldy;
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = col0 + wc * 32 + ct * 16 + 4 * quad + i;
+        if (c < F) {
+          const float g = fminf(product.acc[0][rt][ct][i], limit);
+          const float u = fminf(fmaxf(product.acc[1][rt][ct][i], -limit), limit);
+          dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + 1.0f));
+        }
+      }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void experts_down_tiled_kernel(const T* __restrict__ act, long ldy,
+                                                                 const T* __restrict__ w_down, int N, int F, int top,
+                                                                 int n_tokens, const int* __restrict__ order,
+                                                                 const int* __restrict__ tiles,
+                                                                 const float* __restrict__ weight, float* __restrict__ P) {
+  __shared__ __attribute__((aligned(16))) char lds[2 * 2 * 64 * kLdsRow];
+  const int e = tiles[4 * blockIdx.x];
+  if (e < 0) return;
+  const int first = tiles[4 * blockIdx.x + 1], rows = tiles[4 * blockIdx.x + 2];
+  const int col0 = blockIdx.y * 64;
+  const T* a_row[2];
+  const T* b_row[1][2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int r = (threadIdx.x >> 3) + 32 * j;
+    a_row[j] = r < rows ? act + (long)(first + r) * ldy : nullptr;
+    b_row[0][j] = col0 + r < N ? w_down + ((long)e * N + col0 + r) * F : nullptr;
+  }
+  TiledProduct<T, 1> product;
+  product.run(a_row, b_row, F, lds);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4, wr = w >> 1, wc = w & 1;
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int r = wr * 32 + rt * 16 + l16;
+    if (r >= rows) continue;
+    const int pair = order[first + r];
+    const float share = weight[pair];
+    float* dst = P + ((long)(pair % top) * n_tokens + pair / top) * N;
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = col0 + wc * 32 + ct * 16 + 4 * quad + i;
+        if (c < N) dst[c] = share * product.acc[0][rt][ct][i];
+      }
+  }
+}
+
 }  // namespace ls
 
 LS_DEFINE_ERROR_API
@@ -421,11 +586,25 @@ extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* 
     hipLaunchKernelGGL((experts_down_kernel<T_, RT_, KS_>), grid_down, dim3(256), 0, s, (const T_*)act, ldy,          \
                        (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
   } while (0)
+  // tiles of 64 rows go through LDS where every row of every operand starts on a 16-byte boundary
+  const bool staged = rows_a_tile == 64 && K % vec == 0 && F % vec == 0 && ldx % vec == 0 && ldy % vec == 0;
+#define LS_EXPERTS_STAGED(T_)                                                                                         \
+  do {                                                                                                                \
+    hipLaunchKernelGGL(experts_gate_up_tiled_kernel<T_>, grid_up, dim3(256), 0, s, (const T_*)x, ldx,                 \
+                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, (T_*)act, ldy);     \
+    hipLaunchKernelGGL(experts_down_tiled_kernel<T_>, grid_down, dim3(256), 0, s, (const T_*)act, ldy,                \
+                       (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
+  } while (0)
 #define LS_EXPERTS_BY_ROWS(T_)                 \
   switch (rows_a_tile) {                       \
     case 16: LS_EXPERTS(T_, 1, 4); break;      \
     case 32: LS_EXPERTS(T_, 2, 1); break;      \
-    default: LS_EXPERTS(T_, 4, 1); break;      \
+    default:                                   \
+      if (staged)                              \
+        LS_EXPERTS_STAGED(T_);                 \
+      else                                     \
+        LS_EXPERTS(T_, 4, 1);                  \
+      break;                                   \
   }
   if (dtype == kF32) {
     LS_EXPERTS_BY_ROWS(float)
@@ -433,6 +612,7 @@ extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* 
     LS_EXPERTS_BY_ROWS(bf16_t)
   }
 #undef LS_EXPERTS_BY_ROWS
+#undef LS_EXPERTS_STAGED
 #undef LS_EXPERTS
   return check_launch("experts_apply");
 }

@@ -1,7 +1,7 @@
 """Small Biberax configurations and weights for the tests.  The configurations differ from each
 other in every size and option: numbers of heads (also as many key/value heads as query heads, one
 key/value head, a group of sixteen and more heads), key and value sizes (equal and unequal, also no
-multiples of 16), rotated dimensions (part of the head, all of it, none), frequency scaling (with
+multiples of 16 or of 8), rotated dimensions (part of the head, all of it, none), frequency scaling (with
 all three ranges in use, and none), chunks (shorter than a page, no multiple of a page or a tile,
 longer than any sequence, none), bias tables of several sizes with a farthest distance inside and
 beyond the sequences, experts (one chosen, several, all), layers without a feed-forward or without a
@@ -74,6 +74,12 @@ CASES = {
         routed(rotary(2, 2, 16, 16, chunk=5, rot=16, scale=0.5, scaling=(2.0, 1.0, 2.0, 16)), 16, 1.0, experts=4, top=2,
                shared=(16, 0.5)),
         bare(biased(16, 1, 16, farthest=16, rows=8, scale=0.25)),
+    ])),
+    # key sizes that are no multiple of eight (padded in the cache), value sizes that are no multiple of four, three
+    # query heads on one key/value head, a chunk of eleven, two rows in a bias table
+    "D": dict(page_size=8, raw=config(48, 80, [
+        routed(rotary(3, 1, 20, 6, chunk=11, rot=10, scale=0.2, base=50.0), 12, 1.0, experts=9, top=4, shared=(20, 2.0)),
+        dense(biased(4, 2, 12, farthest=7, rows=2, scale=0.3), 56),
     ])),
 }
 

@@ -258,7 +258,7 @@ def test_small_functions():
     assert torch.allclose(plain.bounded_gated_unit(one, w, "u", 1.5), torch.tensor([[1.5 / (1 + math.exp(-1.702 * 1.5)) * (-1.5 + 1)]], dtype=F64))
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_plain_model_runs_every_case_and_later_tokens_do_not_change_earlier_logits(name):
     raw = CASES[name]["raw"]
     tensors = make_tensors(raw, seed=4)

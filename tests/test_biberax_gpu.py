@@ -321,7 +321,7 @@ def test_each_mechanism_alone_whole_and_in_portions(models, kind, dtype):
         cache.audit()
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_whole_prompt_portions_and_token_by_token_agree_with_the_plain_model(models, name, dtype):
     model, oracle, raw, page, _ = models(name, dtype)
@@ -365,7 +365,7 @@ def test_first_tokens_and_prompts_of_one_and_two_tokens(models, name):
         assert rel_err(feed(model, cache, "r", tokens, []), oracle.forward(tokens)) < TOL["float32"], n
 
 
-@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("C", "float32"), ("A", "bfloat16")])
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("C", "float32"), ("D", "float32"), ("A", "bfloat16")])
 def test_mixed_batches_of_unequal_requests_with_pages_and_slots_used_again(models, name, dtype):
     """Seven requests of unequal lengths through four slots and a pool that holds the live ones only:
     portions beside single tokens, requests that sit steps out, finished requests whose (poisoned)
