@@ -95,6 +95,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
   const int my_head = g * GS + (head_ok ? in_group : 0);
   const int p_first = m.q_start + row0, p_last = p_first + nrows - 1;
   const int* my_table = table + (long)m.table_row * table_stride;
+  const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;   // (pages hold a power of two of keys)
 
   bool row_ok[RT];
   int my_pos[RT], my_lo[RT];
@@ -142,12 +143,12 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int key = key0 + 16 * half + l16;
-      const int page = key <= p_last ? my_table[key / page_size] : -1;
+      const int page = key <= p_last ? my_table[key >> page_shift] : -1;
       const bool k_ok = page >= 0;
-      const long k_at = ((long)(k_ok ? page : 0) * G + g) * page_size + (k_ok ? key % page_size : 0);
+      const long k_at = (((long)(k_ok ? page : 0) * G + g) << page_shift) + (k_ok ? key & page_mask : 0);
       const int key4 = key0 + 16 * half + 4 * quad;
-      const int page4 = key4 <= p_last ? my_table[key4 / page_size] : -1;
-      const long v_at = ((long)(page4 >= 0 ? page4 : 0) * G + g) * DV * page_size + (page4 >= 0 ? key4 % page_size : 0);
+      const int page4 = key4 <= p_last ? my_table[key4 >> page_shift] : -1;
+      const long v_at = ((((long)(page4 >= 0 ? page4 : 0) * G + g) * DV) << page_shift) + (page4 >= 0 ? key4 & page_mask : 0);
       t.v_at[half] = v_at;
 #pragma unroll
       for (int i = 0; i < 4; ++i) t.v_ok[half][i] = page4 >= 0 && key4 + i <= p_last;
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
       if constexpr (kAheadV) {   // (the values too: they are on their way while the scores are formed)
 #pragma unroll
         for (int b = 0; b < VB; ++b) {
-          const long column = (long)(16 * b + l16 < DV ? 16 * b + l16 : 0) * page_size;
+          const long column = (long)(16 * b + l16 < DV ? 16 * b + l16 : 0) << page_shift;
           t.vv[half][b] = *reinterpret_cast<const v4_t*>(v_pages + v_at + column);
         }
       }
@@ -278,11 +279,9 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
       if constexpr (sizeof(T) == 2) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          pb[r][0][i] = (bf16_t)s[r][0][i];
-          pb[r][0][4 + i] = (bf16_t)s[r][1][i];
-        }
+        typedef __attribute__((ext_vector_type(8))) float f32x8;
+        const f32x8 both = __builtin_shufflevector(s[r][0], s[r][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        pb[r][0] = __builtin_convertvector(both, bf16x8);
       } else {
 #pragma unroll
         for (int half = 0; half < 2; ++half)
@@ -293,7 +292,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
 #pragma unroll
     for (int b = 0; b < VB; ++b) {
       const bool col_ok = 16 * b + l16 < DV;
-      const long column = (long)(col_ok ? 16 * b + l16 : 0) * page_size;
+      const long column = (long)(col_ok ? 16 * b + l16 : 0) << page_shift;
       auto value4 = [&](int half) LS_INLINED {
         if constexpr (kAheadV) {
           return vv[half][b];
@@ -305,11 +304,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
         const bf16x4 v0 = value4(0), v1 = value4(1);
         bf16x8 a;
         if (all_held) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            a[i] = v0[i];
-            a[4 + i] = v1[i];
-          }
+          a = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
         } else {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
@@ -461,7 +456,8 @@ extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void*
   LS_REQUIRE(n_items > 0 && q && k_pages && v_pages && table && seqs && items && out, "sink_attention: null operand");
   LS_REQUIRE(H > 0 && G > 0 && H % G == 0, "sink_attention: %d query heads over %d key/value heads", H, G);
   LS_REQUIRE(ldq >= (long)H * D && ldo >= (long)H * DV && (!gate || ldg >= (long)H * DV), "sink_attention: rows are too short");
-  LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && table_stride > 0, "sink_attention: page size %d", page_size);
+  LS_REQUIRE(page_size >= 4 && (page_size & (page_size - 1)) == 0 && table_stride > 0,
+             "sink_attention: page size %d is not a power of two", page_size);
   LS_REQUIRE(window >= 0 && chunk >= 0 && (!dist_bias || n_dist > 0), "sink_attention: window %d, chunk %d, %d distances",
              window, chunk, n_dist);
   LS_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
