@@ -442,6 +442,8 @@ def kernel_digest(model) -> str:
     names = [Path(kernels.core_path).stem] + [Path(p).stem for _, p in sorted(kernels.attention_paths.items())]
     names += [Path(kernels.mixers_path).stem] if kernels.mixers_path else []
     names += [Path(p).stem for _, p in sorted(kernels.talking_paths.items())]
+    names += [Path(p).stem for _, p in sorted(kernels.sink_paths.items())]
+    names += [Path(kernels.experts_path).stem] if kernels.experts_path else []
     return ",".join(n.replace("liblockstep_", "") for n in names)
 
 
