@@ -377,6 +377,298 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
   }
 }
 
+// ---------------------------------------------------------------------------
+// Prompt portions, key and value tiles staged in LDS.  The kernel above spends some 25 vector instructions on
+// every MFMA: addresses and selects for each fragment it takes from global memory, and the row statistics of a
+// tile of only 32 keys.  Here a workgroup of four waves copies a tile of kStagedKeys keys (128 bytes of keys a
+// value column: 64 in bfloat16, 32 in float) into LDS once, with a few 16-byte pieces a thread, and every wave
+// reads its fragments from there at constant offsets.  A wave owns 32 rows of one head; the waves of a workgroup
+// are min(GS, 4) query heads of the key/value head times 4 / min(GS, 4) groups of 32 rows, so a work item names a
+// block of 32, 64 or 128 rows.  The next tile is requested into registers while a tile is worked on.  The
+// arithmetic of a row (scores, statistics, sums) is that of the kernel above with larger tiles.
+// ---------------------------------------------------------------------------
+template <typename T> struct Staged {
+  static constexpr int kKeys = 128 / (int)sizeof(T);                 // keys of a tile
+  static constexpr int kKeyRow = D * (int)sizeof(T) + 16;            // bytes from a key to the next in LDS
+  static constexpr int kValueRow = 128 + 16;                         // bytes from a value column to the next
+  static constexpr int kBytes = kKeys * kKeyRow + DV * kValueRow;
+  static constexpr bool kFits = kBytes <= 64 * 1024 && D % Atom<T>::VEC == 0;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void sink_attention_staged_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
+    const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ items,
+    int H, int G, float scale, int window, int chunk, const float* __restrict__ sink,
+    const float* __restrict__ dist_bias, int n_dist, const float* __restrict__ gate, long ldg, T* __restrict__ out,
+    long ldo, float* __restrict__ part, int part_rows) {
+  typedef typename Atom<T>::vec_t vec_t;
+  typedef typename std::conditional<sizeof(T) == 2, bf16x4, f32x4>::type v4_t;
+  constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
+  constexpr int KCH = D / KC + (D % KC ? 1 : 0);
+  constexpr int TK = Staged<T>::kKeys, NG = TK / 16;              // groups of 16 keys in a tile
+  constexpr int kKeyRow = Staged<T>::kKeyRow, kValueRow = Staged<T>::kValueRow;
+  constexpr int kKeyPieces = TK * (D / VEC), kValuePieces = DV * (TK / VEC);
+  constexpr int KP = (kKeyPieces + 255) / 256, VP = (kValuePieces + 255) / 256;
+  __shared__ __attribute__((aligned(16))) char lds[Staged<T>::kFits ? Staged<T>::kBytes : 16];
+  char* const k_lds = lds;
+  char* const v_lds = lds + TK * kKeyRow;
+
+  const int seq = items[4 * blockIdx.x], rb = items[4 * blockIdx.x + 1];
+  const int run = items[4 * blockIdx.x + 2], n_runs = max(1, items[4 * blockIdx.x + 3]);
+  const SeqMeta m = seqs[seq];
+  const int GS = H / G, g = blockIdx.y;
+  const int HW = GS < 4 ? GS : 4, RG = 4 / HW;                     // heads and groups of 32 rows a workgroup
+  const int block_rows = 32 * RG;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4;
+  const int row0 = rb * block_rows;
+  if (row0 >= m.q_len) return;                                      // (the whole workgroup)
+  const int nrows = min(block_rows, m.q_len - row0);
+  const int p_first = m.q_start + row0, p_last = p_first + nrows - 1;
+  const int* my_table = table + (long)m.table_row * table_stride;
+  const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;
+
+  // this wave's head and rows
+  const int in_group = blockIdx.z * HW + w % HW, rg = w / HW;
+  const int wave_row0 = 32 * rg;
+  const bool active = in_group < GS && rg < RG && wave_row0 < nrows;
+  const int my_head = g * GS + (in_group < GS ? in_group : 0);
+  const int wave_first = p_first + min(wave_row0, nrows - 1), wave_last = p_first + min(wave_row0 + 31, nrows - 1);
+  bool row_ok[2];
+  int my_pos[2], my_lo[2];
+  vec_t qv[2][KCH];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int row = wave_row0 + 16 * r + l16;
+    row_ok[r] = active && row < nrows;
+    my_pos[r] = p_first + (row_ok[r] ? row : 0);
+    my_lo[r] = first_seen(my_pos[r], window, chunk);
+    const T* q_row = q + (long)(m.q_off + row0 + (row_ok[r] ? row : 0)) * ldq + (long)my_head * D;
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) {
+      const bool in = c * KC + VEC * quad + VEC <= D;
+      qv[r][c] = load_or_zero<T>(q_row + (in ? c * KC + VEC * quad : 0), row_ok[r] && in);
+    }
+  }
+  const int wave_lo_last = first_seen(wave_last, window, chunk);
+  const float* my_bias = dist_bias ? dist_bias + (long)my_head * n_dist : nullptr;
+
+  float m_run[2], l_run[2];
+  f32x4 acc[2][VB];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    m_run[r] = kNegSentinel;
+    l_run[r] = 0.f;
+#pragma unroll
+    for (int b = 0; b < VB; ++b) acc[r][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int lo_tile = first_seen(p_first, window, chunk) / TK;
+  const int hi_tile = p_last / TK;
+  const int n_tiles = hi_tile - lo_tile + 1;
+  const int per_run = (n_tiles + n_runs - 1) / n_runs;
+  const int step_begin = run * per_run, step_end = min(n_tiles, (run + 1) * per_run);
+
+  // a thread's pieces of a tile: 16 bytes of a key, and of a value column (VEC consecutive keys, inside one page)
+  vec_t k_piece[KP], v_piece[VP];
+  auto request = [&](int step) LS_INLINED {
+    const int key0 = (lo_tile + step) * TK;
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {
+      const int p = threadIdx.x + 256 * j;
+      const int key = key0 + p / (D / VEC), seg = p % (D / VEC);
+      const bool in = p < kKeyPieces && key <= p_last;
+      const int page = in ? my_table[key >> page_shift] : -1;
+      const long at = (((long)(page >= 0 ? page : 0) * G + g) << page_shift) + (page >= 0 ? key & page_mask : 0);
+      k_piece[j] = load_or_zero<T>(k_pages + at * D + seg * VEC, page >= 0);
+    }
+#pragma unroll
+    for (int j = 0; j < VP; ++j) {
+      const int p = threadIdx.x + 256 * j;
+      const int col = p / (TK / VEC), key = key0 + (p % (TK / VEC)) * VEC;
+      const bool in = p < kValuePieces && key <= p_last;
+      const int page = in ? my_table[key >> page_shift] : -1;
+      const long at = ((((long)(page >= 0 ? page : 0) * G + g) * DV + (in ? col : 0)) << page_shift) + (page >= 0 ? key & page_mask : 0);
+      vec_t v = load_or_zero<T>(v_pages + at, page >= 0);
+      if (key0 + TK - 1 > p_last) {                                  // (only the tile that holds the block's last row:
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)                                //  what lies beyond that row is not held)
+          if (key + i > p_last) v[i] = (T)0.f;
+      }
+      v_piece[j] = v;
+    }
+  };
+  auto store = [&]() LS_INLINED {
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {
+      const int p = threadIdx.x + 256 * j;
+      if (p < kKeyPieces) *reinterpret_cast<vec_t*>(k_lds + (p / (D / VEC)) * kKeyRow + (p % (D / VEC)) * 16) = k_piece[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VP; ++j) {
+      const int p = threadIdx.x + 256 * j;
+      if (p < kValuePieces) *reinterpret_cast<vec_t*>(v_lds + (p / (TK / VEC)) * kValueRow + (p % (TK / VEC)) * 16) = v_piece[j];
+    }
+  };
+
+  if (step_begin < step_end) {
+    request(step_begin);
+    store();
+  }
+  __syncthreads();
+  for (int step = step_begin; step < step_end; ++step) {
+    const int key0 = (lo_tile + step) * TK;
+    if (step + 1 < step_end) request(step + 1);
+    if (active && key0 <= wave_last) {
+      // -- 1. transposed scores of the tile's groups of 16 keys ----------------------------------
+      f32x4 s[2][NG];
+#pragma unroll
+      for (int ng = 0; ng < NG; ++ng) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) s[r][ng] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) {
+          const bool in = c * KC + VEC * quad + VEC <= D;
+          vec_t kf = *reinterpret_cast<const vec_t*>(k_lds + (ng * 16 + l16) * kKeyRow + (in ? c * 64 + quad * 16 : 0));
+          if (!in) kf = Atom<T>::zero();
+#pragma unroll
+          for (int r = 0; r < 2; ++r) Atom<T>::mma(s[r][ng], kf, qv[r][c]);
+        }
+      }
+      // -- 2. scale, bias, mask, online softmax -----------------------------------------------------
+      float shrink[2];
+      bool moved = false;
+      auto softmax_tile = [&](auto whole) LS_INLINED {
+        constexpr bool kWhole = decltype(whole)::value;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          bool see[NG][4];
+          float top = kNegSentinel;
+#pragma unroll
+          for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = key0 + 16 * ng + 4 * quad + i;
+              see[ng][i] = kWhole || (row_ok[r] && key <= my_pos[r] && key >= my_lo[r]);
+              float v = s[r][ng][i] * scale;
+              if (my_bias) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
+              s[r][ng][i] = v;
+              top = fmaxf(top, see[ng][i] ? v : kNegSentinel);
+            }
+          top = quad16_max(top);
+          const float m_new = fmaxf(m_run[r], top);
+          shrink[r] = softmax_exp<T>(m_run[r] - m_new);
+          float sum = 0.f;
+#pragma unroll
+          for (int ng = 0; ng < NG; ++ng)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              s[r][ng][i] = see[ng][i] ? softmax_exp<T>(s[r][ng][i] - m_new) : 0.f;
+              sum = sum + s[r][ng][i];
+            }
+          sum = quad16_sum(sum);
+          l_run[r] = l_run[r] * shrink[r] + sum;
+          m_run[r] = m_new;
+          moved = moved || shrink[r] != 1.0f;
+        }
+      };
+      if (key0 + TK - 1 <= wave_first && key0 >= wave_lo_last)
+        softmax_tile(std::true_type{});
+      else
+        softmax_tile(std::false_type{});
+      // -- 3. values ---------------------------------------------------------------------------
+      if (__all(!moved) == 0) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+          for (int b = 0; b < VB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[r][b][i] = acc[r][b][i] * shrink[r];
+      }
+      constexpr int NC = sizeof(T) == 2 ? NG / 2 : NG;   // chunks of keys of the value product
+      vec_t pb[2][NC];
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          if constexpr (sizeof(T) == 2) {
+            typedef __attribute__((ext_vector_type(8))) float f32x8;
+            const f32x8 both = __builtin_shufflevector(s[r][2 * c], s[r][2 * c + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+            pb[r][c] = __builtin_convertvector(both, bf16x8);
+          } else {
+            pb[r][c] = s[r][c];
+          }
+        }
+#pragma unroll
+      for (int b = 0; b < VB; ++b) {
+        const bool col_ok = 16 * b + l16 < DV;
+        const char* column = v_lds + (col_ok ? 16 * b + l16 : 0) * kValueRow;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          vec_t a;
+          if constexpr (sizeof(T) == 2) {
+            const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(column + ((2 * c) * 16 + 4 * quad) * 2);
+            const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(column + ((2 * c + 1) * 16 + 4 * quad) * 2);
+            a = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+          } else {
+            a = *reinterpret_cast<const f32x4*>(column + (c * 16 + 4 * quad) * 4);
+          }
+          if constexpr (DV % 16 != 0) {
+            if (!col_ok) a = Atom<T>::zero();
+          }
+#pragma unroll
+          for (int r = 0; r < 2; ++r) Atom<T>::mma(acc[r][b], a, pb[r][c]);
+        }
+      }
+    }
+    __syncthreads();                       // every wave has read this tile
+    if (step + 1 < step_end) store();
+    __syncthreads();
+  }
+
+  if (!active) return;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    if (!row_ok[r]) continue;
+    const int row = wave_row0 + 16 * r + l16;
+    if (n_runs > 1) {
+      float* dst = part + (((long)blockIdx.x * part_rows + row) * H + my_head) * (DV + 2);
+#pragma unroll
+      for (int b = 0; b < VB; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (16 * b + 4 * quad + i < DV) dst[16 * b + 4 * quad + i] = acc[r][b][i];
+      if (quad == 0) {
+        dst[DV] = m_run[r];
+        dst[DV + 1] = l_run[r];
+      }
+      continue;
+    }
+    float top = m_run[r], total = l_run[r], keep = 1.0f;
+    if (sink) {
+      const float sv = sink[my_head];
+      top = fmaxf(m_run[r], sv);
+      keep = softmax_exp<T>(m_run[r] - top);
+      total = l_run[r] * keep + softmax_exp<T>(sv - top);
+    }
+    const float inv = keep / total;
+    T* dst = out + (long)(m.q_off + row0 + row) * ldo + (long)my_head * DV;
+    const float* g_row = gate ? gate + (long)(m.q_off + row0 + row) * ldg + (long)my_head * DV : nullptr;
+#pragma unroll
+    for (int b = 0; b < VB; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = 16 * b + 4 * quad + i;
+        if (c < DV) {
+          float v = acc[r][b][i] * inv;
+          if (g_row) v = v * sigmoid_f(g_row[c]);
+          dst[c] = from_f32<T>(v);
+        }
+      }
+  }
+}
+
 // Fold the runs of row blocks: a fold item (first work item, runs, first packed row, rows) names the work items
 // first .. first + runs - 1 of one row block, whose partial results are folded in ascending order for each of its
 // rows; the sink joins the sum and the gate multiplies the result.  One workgroup a (fold item, head, row).
@@ -436,6 +728,16 @@ using namespace ls;
 extern "C" int ls_sink_dim() { return D; }
 extern "C" int ls_sink_vdim() { return DV; }
 extern "C" int ls_sink_max_row_tiles() { return 4; }
+// The staged kernel for prompt portions: keys of a tile (0: this library's sizes do not fit it) and rows of a work
+// item's block for H query heads over G key/value heads.
+extern "C" int ls_sink_staged_keys(int dtype) {
+  if (dtype == kF32) return Staged<float>::kFits ? Staged<float>::kKeys : 0;
+  return Staged<bf16_t>::kFits ? Staged<bf16_t>::kKeys : 0;
+}
+extern "C" int ls_sink_staged_rows(int H, int G) {
+  const int GS = H / (G > 0 ? G : 1);
+  return 32 * (4 / (GS < 4 ? (GS > 0 ? GS : 1) : 4));
+}
 
 // q [T][ldq] (H heads of D); key pages [pages][G][page_size][D], value pages [pages][G][DV][page_size]; table
 // [slots][table_stride]; seqs: the step's requests; items: n_items work items of four ints (request of the step,
@@ -450,11 +752,15 @@ extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void*
                                  int chunk, const float* sink, const float* dist_bias, int n_dist, const float* gate,
                                  long ldg, void* out, long ldo, const int* folds, int n_folds, float* part,
                                  int part_rows, void* stream) {
-  LS_REQUIRE(row_tiles == 0 || row_tiles == 1 || row_tiles == 2 || row_tiles == 4, "sink_attention: %d row tiles", row_tiles);
-  LS_REQUIRE(part_rows == (row_tiles ? 16 * row_tiles : 1), "sink_attention: partial results of %d rows", part_rows);
+  LS_REQUIRE(row_tiles == 0 || row_tiles == 1 || row_tiles == 2 || row_tiles == 4 || row_tiles == 8,
+             "sink_attention: %d row tiles", row_tiles);
+  LS_REQUIRE(H > 0 && G > 0 && H % G == 0, "sink_attention: %d query heads over %d key/value heads", H, G);
+  LS_REQUIRE(part_rows == (row_tiles == 8 ? ls_sink_staged_rows(H, G) : row_tiles ? 16 * row_tiles : 1),
+             "sink_attention: partial results of %d rows", part_rows);
+  LS_REQUIRE(row_tiles != 8 || (ls_sink_staged_keys(dtype) > 0 && page_size % (dtype == kF32 ? 4 : 8) == 0),
+             "sink_attention: the staged kernel does not take these sizes (page size %d)", page_size);
   LS_REQUIRE(n_folds >= 0 && (n_folds == 0 || (part && folds)), "sink_attention: %d fold items need partial results", n_folds);
   LS_REQUIRE(n_items > 0 && q && k_pages && v_pages && table && seqs && items && out, "sink_attention: null operand");
-  LS_REQUIRE(H > 0 && G > 0 && H % G == 0, "sink_attention: %d query heads over %d key/value heads", H, G);
   LS_REQUIRE(ldq >= (long)H * D && ldo >= (long)H * DV && (!gate || ldg >= (long)H * DV), "sink_attention: rows are too short");
   LS_REQUIRE(page_size >= 4 && (page_size & (page_size - 1)) == 0 && table_stride > 0,
              "sink_attention: page size %d is not a power of two", page_size);
@@ -474,12 +780,18 @@ extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void*
                      (const T_*)k_pages, (const T_*)v_pages, page_size, table, table_stride, (const SeqMeta*)seqs,     \
                      items, H, G, scale, window, chunk, sink, dist_bias, n_dist, gate, ldg, (T_*)out, ldo, part,       \
                      part_rows)
+#define LS_SINK_STAGED(T_)                                                                                             \
+  hipLaunchKernelGGL(sink_attention_staged_kernel<T_>, dim3(n_items, G, (GS + 3) / 4), dim3(256), 0, s, (const T_*)q,  \
+                     ldq, (const T_*)k_pages, (const T_*)v_pages, page_size, table, table_stride,                      \
+                     (const SeqMeta*)seqs, items, H, G, scale, window, chunk, sink, dist_bias, n_dist, gate, ldg,      \
+                     (T_*)out, ldo, part, part_rows)
 #define LS_SINK_BY_ROWS(T_)                       \
   switch (row_tiles) {                            \
     case 0: LS_SINK_LAUNCH(T_, 1, true); break;   \
     case 1: LS_SINK_LAUNCH(T_, 1, false); break;  \
     case 2: LS_SINK_LAUNCH(T_, 2, false); break;  \
-    default: LS_SINK_LAUNCH(T_, 4, false); break; \
+    case 4: LS_SINK_LAUNCH(T_, 4, false); break;  \
+    default: LS_SINK_STAGED(T_); break;           \
   }
   if (dtype == kF32) {
     LS_SINK_BY_ROWS(float)
@@ -493,6 +805,7 @@ extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void*
                          folds, sink, gate, ldg, (bf16_t*)out, ldo);
   }
 #undef LS_SINK_BY_ROWS
+#undef LS_SINK_STAGED
 #undef LS_SINK_LAUNCH
   return check_launch("sink_attention");
 }

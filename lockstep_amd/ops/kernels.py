@@ -938,6 +938,19 @@ class Kernels:
             self.sink_paths[shape] = str(path)
         return lib
 
+    #: the value of ``row_tiles`` that asks ``sink_attention`` for its kernel with tiles staged in LDS
+    SINK_STAGED = 8
+
+    def sink_staged_keys(self, dim: int, vdim: int, dtype: torch.dtype) -> int:
+        """Keys of a tile of the staged kernel for prompt portions; 0 where the sizes do not fit it."""
+        return self._memo(("sink_staged_keys", dim, vdim, dtype),
+                          lambda: int(self.sink_lib(dim, vdim).ls_sink_staged_keys(c_int(DTYPE_CODE[dtype]))))
+
+    def sink_staged_rows(self, heads: int, kv_heads: int) -> int:
+        """Rows of a work item's block in the staged kernel: four waves are min(group, 4) heads times groups of 32 rows."""
+        group = heads // kv_heads
+        return 32 * (4 // min(group, 4))
+
     def qkv_post(self, raw: torch.Tensor, n_tokens: int, heads: int, kv_heads: int, dim: int, vdim: int, bias, q_norm,
                  k_norm, eps: float, cos, sin, rot: int, neighbours: bool, max_pos: int, tok_seq, tok_pos, seqs, table,
                  q_out: torch.Tensor, k_pages, v_pages, page_size: int, keys_are_values: bool = False,
@@ -986,7 +999,8 @@ class Kernels:
                        folds: torch.Tensor | None = None, n_folds: int = 0, part: torch.Tensor | None = None) -> None:
         """Attention of the step's queries ``q [T, heads*dim]`` over the paged cache with a sink in the softmax.
         ``items``: ``n_items`` work items of four ints (request of the step, block of ``16 * row_tiles`` of its
-        rows, run, runs); ``row_tiles`` 1, 2 or 4, or 0 for a step of single decoded tokens.  ``window`` /
+        rows, run, runs); ``row_tiles`` 1, 2 or 4, or 0 for a step of single decoded tokens, or ``SINK_STAGED`` for
+        the kernel that stages key tiles in LDS (blocks of ``sink_staged_rows`` rows).  ``window`` /
         ``chunk``: 0 for none.  ``sink [heads]`` float32 or None; ``dist_bias [heads, distances]`` float32 or
         None (its last column serves every larger distance); ``gate``: float32 rows of ``heads*vdim`` logits
         whose sigmoid multiplies the output, or None.  Row blocks whose keys are dealt to several work items
@@ -1000,9 +1014,14 @@ class Kernels:
         self._paged_ok(k_pages, v_pages, table, q.dtype, kv_heads, page_size, dim, vdim)
         if not (items.is_cuda and items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 4 * n_items):
             raise KernelError("sink_attention work items must hold four int32 each")
-        if row_tiles not in (0, 1, 2, 4):
-            raise KernelError(f"sink_attention takes 0, 1, 2 or 4 row tiles, got {row_tiles}")
-        part_rows = 16 * row_tiles if row_tiles else 1
+        if row_tiles not in (0, 1, 2, 4, self.SINK_STAGED):
+            raise KernelError(f"sink_attention takes 0, 1, 2 or 4 row tiles or {self.SINK_STAGED} for its staged kernel, got {row_tiles}")
+        if row_tiles == self.SINK_STAGED:
+            if not (self.sink_staged_keys(dim, vdim, q.dtype) and page_size % (16 // q.element_size()) == 0):
+                raise KernelError(f"the staged kernel does not take keys of {dim}, values of {vdim} on pages of {page_size}")
+            part_rows = self.sink_staged_rows(heads, kv_heads)
+        else:
+            part_rows = 16 * row_tiles if row_tiles else 1
         if n_folds:
             if not (folds is not None and folds.is_cuda and folds.dtype == torch.int32 and folds.is_contiguous()
                     and folds.numel() >= 4 * n_folds and part is not None and part.is_cuda

@@ -38,6 +38,7 @@ MAX_RUNS = 16          # the most runs the keys of a row block are dealt to
 TILES_A_RUN = 8        # a row block of a prompt portion is cut into runs of at least this many tiles
 TILES_A_DECODE_RUN = 2  # ... of a decoded token
 ROW_TILES = int(__import__("os").environ.get("LOCKSTEP_SINK_ROW_TILES", "0"))   # 0: chosen by the step's size
+STAGED = 8             # the value of row_tiles that names the kernel with tiles staged in LDS
 
 
 def distance_buckets(rows: int, farthest: float) -> list[int]:
@@ -180,10 +181,11 @@ class SinkAttention(Mixer):
 
     def prepare_group(self):
         share = getattr(self.position, "share_key", None)
-        return None if share is None else ("sink_attention", self.window, self.chunk, share())
+        return None if share is None else ("sink_attention", self.window, self.chunk, self.nq, self.nkv, self.dk, self.dv, share())
 
     def _block_key(self):
-        return ("sink_attention", "work", self.window, self.chunk)
+        # (the blocks of rows and the tiles of keys depend on the heads and the sizes as well)
+        return ("sink_attention", "work", self.window, self.chunk, self.nq, self.nkv, self.dk, self.dv)
 
     def _first_seen(self, positions):
         lo = np.zeros_like(positions)
@@ -220,19 +222,30 @@ class SinkAttention(Mixer):
             row_tiles = 0
         else:
             longest_portion = int(ctx.q_len.max())
-            # (two row tiles a wave measure best at key sizes of 128: 16.7 ms against 18.1 with one and 17.6 with
-            # four for a prompt of 2,048 tokens at Qwen3-0.6B sizes; four remain for measurements)
-            row_tiles = ROW_TILES or (1 if longest_portion <= 16 else 2)
-            block_rows = 16 * row_tiles
+            kernels = ctx.rt.kernels
+            page = ctx.cache.page_size
+            staged_keys = kernels.sink_staged_keys(self.dk, self.dv, ctx.rt.dtype)
+            # portions of more than 16 tokens: tiles staged in LDS where the sizes fit; else fragments straight from
+            # global memory, two row tiles a wave (one for short portions; four remain for measurements)
+            if ROW_TILES:
+                row_tiles = ROW_TILES
+            elif longest_portion <= 16:
+                row_tiles = 1
+            elif staged_keys and page % (8 if ctx.rt.dtype == torch.bfloat16 else 4) == 0:
+                row_tiles = STAGED
+            else:
+                row_tiles = 2
+            block_rows = kernels.sink_staged_rows(self.nq, self.nkv) if row_tiles == STAGED else 16 * row_tiles
+            tile_keys = staged_keys if row_tiles == STAGED else TILE_KEYS
             counts = -(-ctx.q_len // block_rows)
             seq = np.repeat(np.arange(ctx.n_seqs), counts)
             block = np.arange(int(counts.sum())) - np.repeat(np.cumsum(counts) - counts, counts)
             first = ctx.q_start[seq] + block * block_rows                          # position of a block's first row
             rows = np.minimum(block_rows, ctx.q_len[seq] - block * block_rows)
             last = first + rows - 1
-            tiles = last // TILE_KEYS - self._first_seen(first) // TILE_KEYS + 1    # (as the kernel counts them)
-            # runs of at least TILES_A_RUN tiles, longer where the step has more work than a few items a CU
-            a_run = max(TILES_A_RUN, -(-int(tiles.sum()) * groups // (4 * cus)))
+            tiles = last // tile_keys - self._first_seen(first) // tile_keys + 1    # (as the kernel counts them)
+            # runs of at least TILES_A_RUN tiles of 32 keys, longer where the step has more work than a few items a CU
+            a_run = max(TILES_A_RUN * TILE_KEYS // tile_keys, -(-int(tiles.sum()) * groups // (4 * cus)))
             runs = np.minimum(MAX_RUNS, np.maximum(1, tiles // a_run))
             item_block = np.repeat(np.arange(len(seq)), runs)
             run = np.arange(int(runs.sum())) - np.repeat(np.cumsum(runs) - runs, runs)
@@ -266,7 +279,7 @@ class SinkAttention(Mixer):
         attn = ctx.buf("sink.out", (t, nq * dv), rt.dtype)
         n_items, n_folds, row_tiles = ctx.notes[key]
         work = ctx.block(key)
-        part_rows = 16 * row_tiles if row_tiles else 1
+        part_rows = k.sink_staged_rows(nq, nkv) if row_tiles == STAGED else 16 * row_tiles if row_tiles else 1
         part = ctx.buf("sink.part", (n_items * part_rows * nq * (dv + 2),), torch.float32) if n_folds else None
         gate = raw[:, raw.shape[1] - nq * dv:] if self.gate else None
         k.sink_attention(q, nq, nkv, self.dk, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
