@@ -222,8 +222,8 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
     // whole wave, so the choice costs a scalar branch.
     float shrink[RT];
     bool moved = false;
-    auto softmax_tile = [&](auto whole) LS_INLINED {
-      constexpr bool kWhole = decltype(whole)::value;
+    auto softmax_tile = [&](auto whole, auto biased) LS_INLINED {
+      constexpr bool kWhole = decltype(whole)::value, kBiased = decltype(biased)::value;
 #pragma unroll
       for (int r = 0; r < RT; ++r) {
         bool see[2][4];
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
             const int key = key0 + 16 * half + 4 * quad + i;
             see[half][i] = kWhole || (row_ok[r] && key <= my_pos[r] && key >= my_lo[r]);
             float v = s[r][half][i] * scale;
-            if (my_bias) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
+            if constexpr (kBiased) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
             s[r][half][i] = v;
             top = fmaxf(top, see[half][i] ? v : kNegSentinel);
           }
@@ -256,10 +256,15 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
         moved = moved || shrink[r] != 1.0f;
       }
     };
-    if (key0 + kTileKeys - 1 <= p_first && key0 >= lo_last)
-      softmax_tile(std::true_type{});
-    else
-      softmax_tile(std::false_type{});
+    // (the mask and the bias are instances of the code, chosen by scalar branches once a tile)
+    const bool whole_tile = key0 + kTileKeys - 1 <= p_first && key0 >= lo_last;
+    if (my_bias) {
+      if (whole_tile) softmax_tile(std::true_type{}, std::true_type{});
+      else softmax_tile(std::false_type{}, std::true_type{});
+    } else {
+      if (whole_tile) softmax_tile(std::true_type{}, std::false_type{});
+      else softmax_tile(std::false_type{}, std::false_type{});
+    }
     // -- 3. values: column 16 b + l16 of V^T, keys 4 quad .. 4 quad + 3 of each half ----------------
     bool held = true;
 #pragma unroll
@@ -413,6 +418,10 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
   __shared__ __attribute__((aligned(16))) char lds[Staged<T>::kFits ? Staged<T>::kBytes : 16];
   char* const k_lds = lds;
   char* const v_lds = lds + TK * kKeyRow;
+  // the page ids of a tile and of the next one: looked up by a few threads two tiles ahead, so that no thread waits
+  // for the block table before it can ask for its pieces
+  constexpr int kTilePages = 16;
+  __shared__ int page_s[2][kTilePages];
 
   const int seq = items[4 * blockIdx.x], rb = items[4 * blockIdx.x + 1];
   const int run = items[4 * blockIdx.x + 2], n_runs = max(1, items[4 * blockIdx.x + 3]);
@@ -472,14 +481,24 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
 
   // a thread's pieces of a tile: 16 bytes of a key, and of a value column (VEC consecutive keys, inside one page)
   vec_t k_piece[KP], v_piece[VP];
+  // (pages of at least a tile's keys: one page a tile)
+  const int tile_pages = max(1, TK >> page_shift);
+  auto look_up = [&](int step) LS_INLINED {       // thread i: the page of the tile's i-th run of keys, -1 beyond the block
+    const int key0 = (lo_tile + step) * TK;
+    const int key = max(key0, ((key0 >> page_shift) + (int)threadIdx.x) << page_shift);
+    const bool in = (int)threadIdx.x < tile_pages && step < step_end && key <= p_last;
+    return in ? my_table[key >> page_shift] : -1;
+  };
   auto request = [&](int step) LS_INLINED {
     const int key0 = (lo_tile + step) * TK;
+    const int* pages = page_s[step & 1];
+    const int first_page = key0 >> page_shift;
 #pragma unroll
     for (int j = 0; j < KP; ++j) {
       const int p = threadIdx.x + 256 * j;
       const int key = key0 + p / (D / VEC), seg = p % (D / VEC);
       const bool in = p < kKeyPieces && key <= p_last;
-      const int page = in ? my_table[key >> page_shift] : -1;
+      const int page = in ? pages[(key >> page_shift) - first_page] : -1;
       const long at = (((long)(page >= 0 ? page : 0) * G + g) << page_shift) + (page >= 0 ? key & page_mask : 0);
       k_piece[j] = load_or_zero<T>(k_pages + at * D + seg * VEC, page >= 0);
     }
@@ -488,7 +507,7 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
       const int p = threadIdx.x + 256 * j;
       const int col = p / (TK / VEC), key = key0 + (p % (TK / VEC)) * VEC;
       const bool in = p < kValuePieces && key <= p_last;
-      const int page = in ? my_table[key >> page_shift] : -1;
+      const int page = in ? pages[(key >> page_shift) - first_page] : -1;
       const long at = ((((long)(page >= 0 ? page : 0) * G + g) * DV + (in ? col : 0)) << page_shift) + (page >= 0 ? key & page_mask : 0);
       vec_t v = load_or_zero<T>(v_pages + at, page >= 0);
       if (key0 + TK - 1 > p_last) {                                  // (only the tile that holds the block's last row:
@@ -512,6 +531,11 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
     }
   };
 
+  if (threadIdx.x < kTilePages) {
+    page_s[step_begin & 1][threadIdx.x] = look_up(step_begin);
+    page_s[(step_begin + 1) & 1][threadIdx.x] = look_up(step_begin + 1);
+  }
+  __syncthreads();
   if (step_begin < step_end) {
     request(step_begin);
     store();
@@ -519,6 +543,7 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
   __syncthreads();
   for (int step = step_begin; step < step_end; ++step) {
     const int key0 = (lo_tile + step) * TK;
+    const int page_after = threadIdx.x < kTilePages ? look_up(step + 2) : -1;   // (on its way during the tile)
     if (step + 1 < step_end) request(step + 1);
     if (active && key0 <= wave_last) {
       // -- 1. transposed scores of the tile's groups of 16 keys ----------------------------------
@@ -539,8 +564,8 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
       // -- 2. scale, bias, mask, online softmax -----------------------------------------------------
       float shrink[2];
       bool moved = false;
-      auto softmax_tile = [&](auto whole) LS_INLINED {
-        constexpr bool kWhole = decltype(whole)::value;
+      auto softmax_tile = [&](auto whole, auto biased) LS_INLINED {
+        constexpr bool kWhole = decltype(whole)::value, kBiased = decltype(biased)::value;
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
           bool see[NG][4];
@@ -552,7 +577,7 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
               const int key = key0 + 16 * ng + 4 * quad + i;
               see[ng][i] = kWhole || (row_ok[r] && key <= my_pos[r] && key >= my_lo[r]);
               float v = s[r][ng][i] * scale;
-              if (my_bias) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
+              if constexpr (kBiased) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
               s[r][ng][i] = v;
               top = fmaxf(top, see[ng][i] ? v : kNegSentinel);
             }
@@ -573,10 +598,14 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
           moved = moved || shrink[r] != 1.0f;
         }
       };
-      if (key0 + TK - 1 <= wave_first && key0 >= wave_lo_last)
-        softmax_tile(std::true_type{});
-      else
-        softmax_tile(std::false_type{});
+      const bool whole_tile = key0 + TK - 1 <= wave_first && key0 >= wave_lo_last;
+      if (my_bias) {
+        if (whole_tile) softmax_tile(std::true_type{}, std::true_type{});
+        else softmax_tile(std::false_type{}, std::true_type{});
+      } else {
+        if (whole_tile) softmax_tile(std::true_type{}, std::false_type{});
+        else softmax_tile(std::false_type{}, std::false_type{});
+      }
       // -- 3. values ---------------------------------------------------------------------------
       if (__all(!moved) == 0) {
 #pragma unroll
@@ -624,6 +653,7 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
     }
     __syncthreads();                       // every wave has read this tile
     if (step + 1 < step_end) store();
+    if (threadIdx.x < kTilePages) page_s[step & 1][threadIdx.x] = page_after;   // (this tile's ids are no longer read)
     __syncthreads();
   }
 
